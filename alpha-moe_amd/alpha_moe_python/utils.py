@@ -1,0 +1,59 @@
+"""Layout and tuning-table helpers of the fused W8A8 MoE operator.
+
+Same import path and signatures as the reference's
+``alpha_moe_python/utils.py`` (``interleave_tensor`` at utils.py:5-17,
+``get_best_config`` at utils.py:19-29); the implementations are independent
+restatements of the closed forms.
+"""
+import functools
+import json
+
+import torch
+
+
+def interleave_tensor(tensor: torch.Tensor, rep: int = 8) -> torch.Tensor:
+    """Interleave the gate half and the up half of dim 1 in chunks of ``rep`` rows.
+
+    Input ``[E, N, K]`` holds rows ``[gate_0..gate_{N/2-1}, up_0..up_{N/2-1}]``.
+    Output row ``2*rep*c + h*rep + j`` is input row ``h*(N/2) + rep*c + j``
+    (``h`` = 0 gate / 1 up, ``c`` = chunk, ``j`` < rep).  Weights use rep=8,
+    128x128 block scales use rep=1 (reference utils.py:5-17).
+    """
+    if tensor.dim() != 3:
+        raise ValueError(f"interleave_tensor expects [E, N, K], got {tuple(tensor.shape)}")
+    E, N, K = tensor.shape
+    if rep <= 0 or N % (2 * rep) != 0:
+        raise ValueError(f"N={N} must be a multiple of 2*rep={2 * rep}")
+    chunks = N // (2 * rep)
+    # [E, half, chunk, j, K] -> [E, chunk, half, j, K]
+    return tensor.reshape(E, 2, chunks, rep, K).permute(0, 2, 1, 3, 4).reshape(E, N, K).contiguous()
+
+
+def deinterleave_tensor(tensor: torch.Tensor, rep: int = 8) -> torch.Tensor:
+    """Inverse of :func:`interleave_tensor` (no counterpart in the reference; used by tests and tools)."""
+    if tensor.dim() != 3:
+        raise ValueError(f"deinterleave_tensor expects [E, N, K], got {tuple(tensor.shape)}")
+    E, N, K = tensor.shape
+    if rep <= 0 or N % (2 * rep) != 0:
+        raise ValueError(f"N={N} must be a multiple of 2*rep={2 * rep}")
+    chunks = N // (2 * rep)
+    return tensor.reshape(E, chunks, 2, rep, K).permute(0, 2, 1, 3, 4).reshape(E, N, K).contiguous()
+
+
+@functools.lru_cache()
+def get_best_config(path: str, n_tokens: int):
+    """Entry of the JSON tuning table whose integer key is nearest to ``n_tokens``.
+
+    The table maps ``str(M)`` to ``{"block_m", "block_n", "warp_n", "stages"}``.
+    Ties go to the key that comes first in the file; results are memoised per
+    ``(path, n_tokens)`` (reference utils.py:19-29).
+    """
+    with open(path, "r") as fh:
+        table = json.load(fh)
+    best = None
+    best_dist = None
+    for key, cfg in table.items():
+        dist = abs(int(key) - n_tokens)
+        if best_dist is None or dist < best_dist:
+            best, best_dist = cfg, dist
+    return best

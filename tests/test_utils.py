@@ -1,0 +1,79 @@
+"""interleave_tensor / get_best_config against closed forms, brute force and the reference's shipped tables."""
+import json
+import os
+
+import pytest
+import torch
+
+from alpha_moe_python.utils import deinterleave_tensor, get_best_config, interleave_tensor
+from oracle import moe_oracle as O
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "ref_config_entries.json")
+
+
+@pytest.mark.parametrize("rep", [1, 2, 8])
+@pytest.mark.parametrize("shape", [(2, 32, 3), (1, 16, 5), (3, 256, 4)])
+def test_interleave_matches_index_loop(shape, rep):
+    t = torch.arange(shape[0] * shape[1] * shape[2], dtype=torch.float32).reshape(shape)
+    got = interleave_tensor(t, rep)
+    assert got.is_contiguous()
+    assert torch.equal(got, O.interleave_reference(t, rep))
+    assert torch.equal(deinterleave_tensor(got, rep), t)
+    assert torch.equal(O.deinterleave_reference(got, rep), t)
+
+
+def test_interleave_row_pattern_of_readme():
+    # README.md:96-102 of the reference: g0..g7,u0..u7,g8..g15,u8..u15,...
+    N = 32
+    t = torch.arange(N).reshape(1, N, 1)
+    got = interleave_tensor(t, 8).flatten().tolist()
+    g, u = list(range(0, 16)), list(range(16, 32))
+    assert got == g[0:8] + u[0:8] + g[8:16] + u[8:16]
+    # scales, rep=1: gs0,us0,gs1,us1
+    s = torch.arange(4).reshape(1, 4, 1)
+    assert interleave_tensor(s, 1).flatten().tolist() == [0, 2, 1, 3]
+
+
+def test_interleave_dtypes_and_errors():
+    w = torch.randn(2, 32, 128).to(torch.float8_e4m3fn)
+    got = interleave_tensor(w, 8)
+    assert got.dtype == torch.float8_e4m3fn
+    assert torch.equal(got.view(torch.uint8), O.interleave_reference(w.view(torch.uint8), 8))
+    with pytest.raises(ValueError):
+        interleave_tensor(torch.zeros(1, 24, 4), 8)
+    with pytest.raises(ValueError):
+        interleave_tensor(torch.zeros(24, 4), 8)
+
+
+def test_get_best_config_nearest_and_ties(tmp_path):
+    table = {"1": {"block_m": 16, "block_n": 32, "warp_n": 8, "stages": 5},
+             "8": {"block_m": 8, "block_n": 32, "warp_n": 8, "stages": 4},
+             "64": {"block_m": 8, "block_n": 64, "warp_n": 4, "stages": 2}}
+    p = tmp_path / "t.json"
+    p.write_text(json.dumps(table))
+    path = str(p)
+    assert get_best_config(path, 1) == table["1"]
+    assert get_best_config(path, 4) == table["1"]       # |1-4|=3 < |8-4|=4
+    assert get_best_config(path, 5) == table["8"]
+    assert get_best_config(path, 36) == table["8"]      # tie 28/28: first key in file order wins
+    assert get_best_config(path, 37) == table["64"]
+    assert get_best_config(path, 10 ** 6) == table["64"]
+    # memoised per (path, n_tokens): a rewritten file is not re-read for a cached query
+    p.write_text(json.dumps({"1": {"block_m": 128, "block_n": 64, "warp_n": 4, "stages": 1}}))
+    assert get_best_config(path, 1) == table["1"]
+    assert get_best_config(path, 2)["block_m"] == 128
+
+
+def test_get_best_config_on_reference_tables(tmp_path):
+    golden = json.load(open(GOLDEN))
+    ds = golden["moe_jit_257_256_7168.json"]
+    assert ds["n_keys"] == 48
+    p = tmp_path / "ds.json"
+    p.write_text(json.dumps(ds["entries"]))
+    assert get_best_config(str(p), 1) == {"block_m": 16, "block_n": 32, "warp_n": 8, "stages": 5}
+    assert get_best_config(str(p), 8192) == {"block_m": 72, "block_n": 32, "warp_n": 8, "stages": 5}
+    assert get_best_config(str(p), 60) == ds["entries"]["64"]
+    assert get_best_config(str(p), 3000) == ds["entries"]["2048"]
+    for cfg in ds["entries"].values():
+        assert set(cfg) == {"block_m", "block_n", "warp_n", "stages"}
+        assert cfg["block_n"] * cfg["warp_n"] == 256
