@@ -1,0 +1,98 @@
+// PyTorch-ROCm binding of the fused W8A8 MoE operator: registers
+// torch.ops.alpha_moe.fused_moe_w8a8_up_down with the schema of the reference
+// (csrc/torch_interface.cpp:105-125), checks the arguments, and forwards raw device pointers plus the
+// current HIP stream to the C ABI in include/alpha_moe_hip.h.  No kernel code lives here.
+//
+// Differences from the reference binding (csrc/torch_interface.cpp:37-103), all on the strict side:
+//   * dtype, device and shape of every tensor are checked (the reference checks contiguity only);
+//   * the device guard is installed before the stream is fetched;
+//   * a refused launch or an unsupported knob raises instead of printing or doing nothing.
+#include <ATen/ATen.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/library.h>
+
+#include "../../include/alpha_moe_hip.h"
+
+namespace {
+
+void check_tensor(const at::Tensor &t, const char *name, at::ScalarType dtype, const at::Device &dev)
+{
+    TORCH_CHECK(t.defined(), name, " is undefined");
+    TORCH_CHECK(t.device() == dev, name, " must be on ", dev, ", got ", t.device());
+    TORCH_CHECK(t.scalar_type() == dtype, name, " must have dtype ", dtype, ", got ", t.scalar_type());
+    TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
+}
+
+void fused_moe_w8a8_up_down(const at::Tensor &x, const at::Tensor &x_scale, const at::Tensor &w,
+                            const at::Tensor &w_scale, const at::Tensor &w2, const at::Tensor &w2_scale,
+                            const at::Tensor &sorted_token_ids, const at::Tensor &expert_ids,
+                            const at::Tensor &num_tokens_post_padded, const at::Tensor &topk_weights,
+                            at::Tensor &out, int64_t top_k, int64_t block_m, int64_t block_n, int64_t warp_n,
+                            int64_t stages, double scaling_factor)
+{
+    TORCH_CHECK(x.is_cuda(), "x must be a GPU tensor");
+    const at::Device dev = x.device();
+    check_tensor(x, "x", at::kFloat8_e4m3fn, dev);
+    check_tensor(x_scale, "x_scale", at::kFloat, dev);
+    check_tensor(w, "w", at::kFloat8_e4m3fn, dev);
+    check_tensor(w_scale, "w_scale", at::kFloat, dev);
+    check_tensor(w2, "w2", at::kFloat8_e4m3fn, dev);
+    check_tensor(w2_scale, "w2_scale", at::kFloat, dev);
+    check_tensor(sorted_token_ids, "sorted_token_ids", at::kInt, dev);
+    check_tensor(expert_ids, "expert_ids", at::kInt, dev);
+    check_tensor(num_tokens_post_padded, "num_tokens_post_padded", at::kInt, dev);
+    check_tensor(topk_weights, "topk_weights", at::kFloat, dev);
+    check_tensor(out, "out", at::kBFloat16, dev);
+
+    TORCH_CHECK(x.dim() == 2 && x.size(0) > 0, "x must be [M, K] with M > 0");
+    const int64_t M = x.size(0), K = x.size(1);
+    TORCH_CHECK(K % 128 == 0, "K dimension must be a multiple of 128");
+    TORCH_CHECK(w.dim() == 3 && w.size(2) == K, "w must be [E, N, K] with the K of x");
+    const int64_t E = w.size(0), N = w.size(1);
+    TORCH_CHECK(N % 256 == 0, "N (= 2 * intermediate size) must be a multiple of 256");
+    TORCH_CHECK(w2.dim() == 3 && w2.size(0) == E && w2.size(1) == K && w2.size(2) == N / 2, "w2 must be [E, K, N/2]");
+    TORCH_CHECK(x_scale.numel() == M * (K / 128), "x_scale must be [M, K/128]");
+    TORCH_CHECK(w_scale.numel() == E * (N / 128) * (K / 128), "w_scale must be [E, N/128, K/128]");
+    TORCH_CHECK(w2_scale.numel() == E * (K / 128) * (N / 256), "w2_scale must be [E, K/128, N/256]");
+    TORCH_CHECK(out.dim() == 2 && out.size(0) == M && out.size(1) == K, "out must be [M, K]");
+    TORCH_CHECK(top_k > 0 && topk_weights.numel() == M * top_k, "topk_weights must hold M * top_k values");
+    TORCH_CHECK((block_n == 64 && warp_n == 4) || (block_n == 32 && warp_n == 8),
+                "(block_n, warp_n) must be (64, 4) or (32, 8)");
+    TORCH_CHECK(stages > 0 && stages < 6, "stages must be in [1, 5]");
+    TORCH_CHECK(block_m > 0 && block_m <= 128 && block_m % 8 == 0, "block_m must be a multiple of 8 in [8, 128]");
+    const int64_t sorted_num = sorted_token_ids.numel();
+    TORCH_CHECK(sorted_num > 0, "sorted_token_ids is empty");
+    TORCH_CHECK(expert_ids.numel() >= (sorted_num + block_m - 1) / block_m,
+                "expert_ids must hold one entry per block_m rows of sorted_token_ids");
+    TORCH_CHECK(num_tokens_post_padded.numel() >= 1, "num_tokens_post_padded must hold one value");
+    TORCH_CHECK(M * top_k <= INT32_MAX && sorted_num <= INT32_MAX && E <= INT32_MAX, "sizes exceed int32");
+
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(dev);
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+
+    const int rc = alpha_moe_fused_moe_w8a8_up_down(
+        static_cast<const uint8_t *>(x.const_data_ptr()), x_scale.const_data_ptr<float>(),
+        static_cast<const uint8_t *>(w.const_data_ptr()), w_scale.const_data_ptr<float>(),
+        static_cast<const uint8_t *>(w2.const_data_ptr()), w2_scale.const_data_ptr<float>(),
+        static_cast<uint16_t *>(out.data_ptr()), sorted_token_ids.const_data_ptr<int32_t>(),
+        expert_ids.const_data_ptr<int32_t>(), num_tokens_post_padded.const_data_ptr<int32_t>(),
+        topk_weights.const_data_ptr<float>(), static_cast<int>(top_k), static_cast<int>(M), static_cast<int>(K),
+        static_cast<int>(N), static_cast<int>(E), static_cast<int>(sorted_num), static_cast<int>(block_m),
+        static_cast<int>(block_n), static_cast<int>(warp_n), static_cast<int>(stages),
+        static_cast<float>(scaling_factor), static_cast<void *>(stream));
+    TORCH_CHECK(rc == ALPHA_MOE_OK, "alpha_moe_fused_moe_w8a8_up_down failed: ", alpha_moe_status_string(rc));
+}
+
+}  // namespace
+
+TORCH_LIBRARY_FRAGMENT(alpha_moe, m)
+{
+    m.def("fused_moe_w8a8_up_down("
+          "Tensor x, Tensor x_scale, Tensor w, Tensor w_scale, Tensor w2, Tensor w2_scale, "
+          "Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_post_padded, Tensor topk_weights, "
+          "Tensor(a!) out, int top_k, int block_m, int block_n, int warp_n, int stages, float scaling_factor"
+          ") -> ()");
+    // GPU tensors of PyTorch-ROCm carry the dispatch key named CUDA
+    m.impl("fused_moe_w8a8_up_down", c10::DispatchKey::CUDA, &fused_moe_w8a8_up_down);
+}

@@ -1,0 +1,79 @@
+/*
+ * C ABI of the MI355X (gfx950) fused W8A8 MoE operator: libalpha_moe_hip.so.
+ *
+ * Plain pointers and sizes only; no torch types.  Every pointer is DEVICE memory, borrowed for the
+ * duration of the enqueued work; nothing is allocated, freed or synchronised; the call is asynchronous on
+ * `stream` and can be captured into a HIP graph.  No function here prints or exits: each returns a status.
+ */
+#ifndef ALPHA_MOE_HIP_H
+#define ALPHA_MOE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum alpha_moe_status {
+    ALPHA_MOE_OK = 0,
+    ALPHA_MOE_ERR_NULL_POINTER = 1,   /* a required pointer is null */
+    ALPHA_MOE_ERR_SHAPE = 2,          /* M<=0, K%128!=0, N%256!=0, top_k<=0, sizes overflow int32 ... */
+    ALPHA_MOE_ERR_BLOCK_M = 3,        /* block_m not in {8,16,...,128} */
+    ALPHA_MOE_ERR_BLOCK_N_WARP_N = 4, /* (block_n, warp_n) not (64,4) or (32,8) */
+    ALPHA_MOE_ERR_STAGES = 5,         /* stages not in 1..5 */
+    ALPHA_MOE_ERR_LAUNCH = 6          /* the HIP runtime refused the launch (see hipGetLastError) */
+};
+
+/*
+ * out[t, :] += scaling_factor * sum_s topk_weights[t, s] * W2_e . requant(SwiGLU(W1_e . x_t)),  e = expert of slot (t, s).
+ *
+ * Replaces the reference's C++ seam `fused_moe_w8a8_wgmma_up_down_acc`
+ * (declared csrc/torch_interface.cpp:12-34, defined
+ * csrc/kernels/fused_moe_w8a8/fused_moe_w8a8_up_down_acc.cu:1258-1303): same parameters in the same order, with
+ * fp8 as uint8_t codes (OCP e4m3fn), bf16 as uint16_t, the stream as an opaque hipStream_t, and an int status
+ * instead of stderr prints / exit().
+ *
+ *   x                [M, K]            fp8, row-major, K % 128 == 0
+ *   x_scale          [M, K/128]        f32, per token per 128 columns
+ *   w                [E, N, K]         fp8, N = 2*I, gate/up rows interleaved in chunks of 8, N % 256 == 0
+ *   w_scale          [E, N/128, K/128] f32, gate/up rows interleaved in chunks of 1
+ *   w2               [E, K, N/2]       fp8
+ *   w2_scale         [E, K/128, N/256] f32
+ *   out              [M, K]            bf16, the result is ADDED (packed bf16 atomics); caller zero-fills
+ *   sorted_token_ids [sorted_num]      flat slot ids t*top_k+s grouped by expert in blocks of block_m; ids >= M*top_k are padding
+ *   expert_ids       [ceil(sorted_num/block_m)]  expert of each block (blocks with an id outside [0,E) are skipped)
+ *   num_tokens_post_padded [1]         blocks starting at or past this row are skipped
+ *   topk_weights     [M*top_k]         f32, indexed by the flat slot id
+ *   block_m          8..128 step 8     must equal the block size sorted_token_ids was built with
+ *   (block_n, warp_n) (64,4) or (32,8) wavefronts per workgroup = warp_n, w1 rows per wavefront = block_n
+ *   stages           1..5              K-blocks of loads kept in flight per wavefront
+ */
+int alpha_moe_fused_moe_w8a8_up_down(
+    const uint8_t *x, const float *x_scale,
+    const uint8_t *w, const float *w_scale,
+    const uint8_t *w2, const float *w2_scale,
+    uint16_t *out,
+    const int32_t *sorted_token_ids, const int32_t *expert_ids, const int32_t *num_tokens_post_padded,
+    const float *topk_weights,
+    int top_k, int M, int K, int N, int num_experts, int sorted_num,
+    int block_m, int block_n, int warp_n, int stages,
+    float scaling_factor, void *stream /* hipStream_t */);
+
+/*
+ * The argument checks of the call above without touching the device: returns the status the launch would
+ * return for these sizes and knobs.  Replaces the knob dispatch of fused_moe_w8a8_up_down_acc.cu:1200-1256,1282-1302
+ * (which prints to stderr and silently does nothing) and the TORCH_CHECKs of torch_interface.cpp:59-64.
+ */
+int alpha_moe_validate(int top_k, int M, int K, int N, int num_experts, int sorted_num,
+                       int block_m, int block_n, int warp_n, int stages);
+
+/* Human-readable text for a status code (static storage). */
+const char *alpha_moe_status_string(int status);
+
+/* Library version, "major.minor". */
+const char *alpha_moe_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ALPHA_MOE_HIP_H */

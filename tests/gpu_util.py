@@ -1,0 +1,50 @@
+"""Shared helpers of the GPU parity tests: run the operator (through torch.ops or straight through the C ABI)
+and the CPU oracle on the same bits."""
+import torch
+
+from oracle import moe_oracle as O
+
+# north-star bar for the bf16 output: max |err| <= 1e-2 * max |ref| and cosine >= 0.9999
+# (accumulation order of the bf16 atomics differs from run to run); routing/indexing is bit-exact.
+MAX_ABS_OVER_MAX_REF = 1e-2
+MIN_COSINE = 0.9999
+
+
+def run_op(P, block_m, block_n, warp_n, stages, out=None, scaling=None, via="torch"):
+    import alpha_moe
+    W = P.weights
+    s_ids, e_ids, total = P.align(block_m)
+    if out is None:
+        out = torch.zeros((P.M, P.shape.K), dtype=torch.bfloat16, device=P.x.device)
+    scaling = P.shape.scaling_factor if scaling is None else scaling
+    if via == "torch":
+        torch.ops.alpha_moe.fused_moe_w8a8_up_down(P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids,
+                                                   total, P.topk_weights, out, P.shape.top_k, block_m, block_n, warp_n,
+                                                   stages, scaling)
+    else:
+        stream = torch.cuda.current_stream().cuda_stream
+        rc = alpha_moe.c_abi.alpha_moe_fused_moe_w8a8_up_down(
+            P.x.data_ptr(), P.x_scale.data_ptr(), W.w1.data_ptr(), W.w1_scale.data_ptr(), W.w2.data_ptr(),
+            W.w2_scale.data_ptr(), out.data_ptr(), s_ids.data_ptr(), e_ids.data_ptr(), total.data_ptr(),
+            P.topk_weights.data_ptr(), P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E, s_ids.numel(), block_m,
+            block_n, warp_n, stages, float(scaling), stream)
+        assert rc == 0, alpha_moe.c_abi.alpha_moe_status_string(rc)
+    torch.cuda.synchronize()
+    return out
+
+
+def oracle_out(P, block_m=16, out=None, scaling=None):
+    W = P.weights
+    s_ids, e_ids, total = P.align(block_m)
+    if out is None:
+        out = torch.zeros((P.M, P.shape.K), dtype=torch.bfloat16)
+    scaling = P.shape.scaling_factor if scaling is None else scaling
+    return O.fused_moe_oracle(P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids, total,
+                              P.topk_weights, out, P.shape.top_k, block_m, scaling)
+
+
+def assert_parity(out, ref, what=""):
+    m = O.error_metrics(out, ref)
+    assert torch.isfinite(out.float()).all(), what
+    assert m["max_abs_over_max_ref"] <= MAX_ABS_OVER_MAX_REF and m["cosine"] >= MIN_COSINE, (what, m)
+    return m

@@ -1,0 +1,108 @@
+"""GPU parity: the HIP operator against the CPU oracle on the same seeded bits.
+
+Bar (written out in gpu_util.py): max |err| / max |ref| <= 1e-2 and cosine >= 0.9999 on the bf16 output.
+"""
+import pytest
+import torch
+
+from alpha_moe_python.workloads import SHAPES, Shape, make_problem, make_weights
+from gpu_util import assert_parity, oracle_out, run_op
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+ALL_KNOBS = [(bm, bn, wn, st) for bm in range(8, 129, 8) for (bn, wn) in ((64, 4), (32, 8)) for st in range(1, 6)]
+
+
+@pytest.fixture(scope="module")
+def c1():
+    W = make_weights(SHAPES["c1"], device=DEV, seed=0)
+    P = make_problem(W, 16, seed=0)
+    return P, oracle_out(P)
+
+
+def test_c1_default_knobs_torch_op_and_c_abi(c1):
+    P, ref = c1
+    print("case c1 M=16 block_m=16 (64,4) stages=3", flush=True)
+    assert_parity(run_op(P, 16, 64, 4, 3, via="torch"), ref, "torch op")
+    assert_parity(run_op(P, 16, 64, 4, 3, via="c_abi"), ref, "c abi")
+
+
+def test_c1_result_independent_of_every_knob(c1):
+    """The reference's correctness sweep runs every (block_m, block_n/warp_n, stages) it accepts
+    (test_moe_correctness.py:172-190); the result may not depend on them."""
+    P, ref = c1
+    for bm, bn, wn, st in ALL_KNOBS:
+        print(f"case c1 M=16 knobs {(bm, bn, wn, st)}", flush=True)
+        assert_parity(run_op(P, bm, bn, wn, st), ref, f"knobs {(bm, bn, wn, st)}")
+
+
+def test_add_semantics_scaling_and_zero_weights(c1):
+    P, ref = c1
+    pre = torch.full((P.M, P.shape.K), 0.25, dtype=torch.bfloat16, device=DEV)
+    got = run_op(P, 16, 32, 8, 2, out=pre.clone())
+    assert_parity(got, oracle_out(P, out=pre.cpu()), "out pre-filled")
+    assert_parity(run_op(P, 16, 64, 4, 2, scaling=2.5), oracle_out(P, scaling=2.5), "scaling 2.5")
+    saved = P.topk_weights
+    P.topk_weights = torch.zeros_like(saved)
+    assert float(run_op(P, 16, 64, 4, 2).float().abs().max()) == 0.0
+    P.topk_weights = saved
+
+
+@pytest.mark.parametrize("M,E,top_k,K,I", [(1, 4, 2, 128, 128), (3, 5, 3, 384, 256), (37, 3, 2, 256, 384), (200, 2, 1, 128, 128)])
+def test_ragged_small_shapes(M, E, top_k, K, I):
+    """K a single block, K % 256 == 128 (the reference silently drops the last 128 columns there), more I blocks,
+    more tokens than one block, experts without tokens."""
+    shape = Shape("t", E=E, top_k=top_k, K=K, I=I, shared_expert=False, routing="softmax_renorm", scaling_factor=1.3,
+                  w_std=0.05)
+    W = make_weights(shape, device=DEV, seed=M)
+    P = make_problem(W, M, seed=M)
+    ref = oracle_out(P)
+    for bm, bn, wn, st in [(8, 64, 4, 1), (16, 32, 8, 5), (48, 64, 4, 3), (128, 32, 8, 2)]:
+        print(f"case ragged {(M, E, top_k, K, I)} knobs {(bm, bn, wn, st)}", flush=True)
+        assert_parity(run_op(P, bm, bn, wn, st), ref, f"{(M, E, top_k, K, I)} knobs {(bm, bn, wn, st)}")
+
+
+def test_duplicate_experts_and_negative_scales():
+    """Duplicate expert ids inside one token's top-k and negative block scales are legal inputs
+    (test_moe_correctness.py:42,59-60 of the reference generates both)."""
+    shape = Shape("t", E=6, top_k=4, K=256, I=128, shared_expert=False, routing="softmax_renorm", scaling_factor=2.5,
+                  w_std=0.05)
+    W = make_weights(shape, device=DEV, seed=3)
+    W.w1_scale.mul_(torch.where(torch.rand_like(W.w1_scale) < 0.5, -1.0, 1.0))
+    W.w2_scale.mul_(torch.where(torch.rand_like(W.w2_scale) < 0.5, -1.0, 1.0))
+    P = make_problem(W, 24, seed=3)
+    g = torch.Generator(device=DEV).manual_seed(7)
+    P.topk_ids = torch.randint(0, 6, (24, 4), generator=g, device=DEV, dtype=torch.int32)   # with replacement
+    P.aligned.clear()
+    ref = oracle_out(P)
+    for bm, bn, wn, st in [(8, 32, 8, 3), (32, 64, 4, 2)]:
+        print(f"case dup/neg knobs {(bm, bn, wn, st)}", flush=True)
+        assert_parity(run_op(P, bm, bn, wn, st), ref, f"dup/neg knobs {(bm, bn, wn, st)}")
+
+
+def test_bad_arguments_raise(c1):
+    P, _ = c1
+    with pytest.raises(RuntimeError):
+        run_op(P, 12, 64, 4, 2)
+    with pytest.raises(RuntimeError):
+        run_op(P, 16, 64, 8, 2)
+    with pytest.raises(RuntimeError):
+        run_op(P, 16, 64, 4, 6)
+    with pytest.raises(RuntimeError):
+        run_op(P, 16, 64, 4, 2, out=torch.zeros((P.M, P.shape.K), dtype=torch.float16, device=DEV))
+
+
+@pytest.fixture(scope="module")
+def ds_weights():
+    return make_weights(SHAPES["ds"], device=DEV, seed=0)
+
+
+@pytest.mark.parametrize("M,knobs", [(1, (16, 32, 8, 5)), (4, (16, 64, 4, 4)), (16, (16, 64, 4, 3)), (64, (16, 32, 8, 3)),
+                                     (64, (8, 64, 4, 2))])
+def test_deepseek_shard_decode_full_size(ds_weights, M, knobs):
+    """BASELINE decode configuration at its real size: E=257, top_k=9, K=7168, I=256."""
+    P = make_problem(ds_weights, M, seed=0)
+    print(f"case ds M={M} knobs {knobs}", flush=True)
+    m = assert_parity(run_op(P, *knobs), oracle_out(P), f"ds M={M} knobs {knobs}")
+    print("metrics", m, flush=True)
