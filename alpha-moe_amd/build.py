@@ -39,8 +39,8 @@ def run(cmd):
 
 
 def build_hip():
-    src = os.path.join(CSRC, "fused_moe_w8a8.hip")
-    run([HIPCC, *HIP_FLAGS, "-o", HIP_LIB, src])
+    srcs = [os.path.join(CSRC, f) for f in ("moe_api.hip", "moe_direct.hip", "moe_stream.hip")]
+    run([HIPCC, *HIP_FLAGS, "-o", HIP_LIB, *srcs])
     return HIP_LIB
 
 

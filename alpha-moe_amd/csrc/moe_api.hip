@@ -1,0 +1,106 @@
+// C ABI of libalpha_moe_hip.so (include/alpha_moe_hip.h): argument checks, kernel-family choice, launches.
+#include <stdlib.h>
+#include <string.h>
+
+#include "moe_common.hpp"
+
+using namespace alpha_moe;
+
+namespace {
+
+// ALPHA_MOE_PATH=direct|stream forces one kernel family (for experiments); default: streaming kernel where it applies.
+int forced_path()
+{
+    static const int v = [] {
+        const char *e = getenv("ALPHA_MOE_PATH");
+        if (!e) return 0;
+        if (!strcmp(e, "direct")) return 1;
+        if (!strcmp(e, "stream")) return 2;
+        return 0;
+    }();
+    return v;
+}
+
+bool use_stream(int block_m)
+{
+    if (!stream_supported(block_m)) return false;
+    return forced_path() != 1;
+}
+
+}  // namespace
+
+extern "C" int alpha_moe_validate(int top_k, int M, int K, int N, int num_experts, int sorted_num, int block_m,
+                                  int block_n, int warp_n, int stages)
+{
+    if (M <= 0 || K <= 0 || N <= 0 || num_experts <= 0 || top_k <= 0 || sorted_num <= 0) return ALPHA_MOE_ERR_SHAPE;
+    if (K % 128 != 0 || N % 256 != 0 || K > 128 * kMaxKBlocks) return ALPHA_MOE_ERR_SHAPE;
+    if ((int64_t)M * top_k > INT32_MAX || (int64_t)M * K / 4 > INT32_MAX) return ALPHA_MOE_ERR_SHAPE;
+    if (block_m < 8 || block_m > 128 || block_m % 8 != 0) return ALPHA_MOE_ERR_BLOCK_M;
+    if (!((block_n == 64 && warp_n == 4) || (block_n == 32 && warp_n == 8))) return ALPHA_MOE_ERR_BLOCK_N_WARP_N;
+    if (stages < 1 || stages > 5) return ALPHA_MOE_ERR_STAGES;
+    const int64_t n_blocks = ((int64_t)sorted_num + block_m - 1) / block_m;
+    if (n_blocks * (N / 256) * (K / 128) > INT32_MAX) return ALPHA_MOE_ERR_SHAPE;
+    return ALPHA_MOE_OK;
+}
+
+extern "C" size_t alpha_moe_workspace_bytes(int M, int K, int N, int sorted_num, int block_m)
+{
+    if (M <= 0 || K <= 0 || N <= 0 || sorted_num <= 0 || block_m <= 0) return 0;
+    const size_t direct = (size_t)M * (size_t)K * sizeof(float);
+    const size_t stream = stream_supported(block_m) ? stream_workspace_bytes(M, K, N, sorted_num, block_m) : 0;
+    return direct > stream ? direct : stream;
+}
+
+extern "C" int alpha_moe_fused_moe_w8a8_up_down(const uint8_t *x, const float *x_scale, const uint8_t *w,
+                                                const float *w_scale, const uint8_t *w2, const float *w2_scale,
+                                                uint16_t *out, const int32_t *sorted_token_ids,
+                                                const int32_t *expert_ids, const int32_t *num_tokens_post_padded,
+                                                const float *topk_weights, int top_k, int M, int K, int N,
+                                                int num_experts, int sorted_num, int block_m, int block_n, int warp_n,
+                                                int stages, float scaling_factor, void *workspace,
+                                                size_t workspace_bytes, void *stream)
+{
+    if (!x || !x_scale || !w || !w_scale || !w2 || !w2_scale || !out || !sorted_token_ids || !expert_ids ||
+        !num_tokens_post_padded || !topk_weights)
+        return ALPHA_MOE_ERR_NULL_POINTER;
+    const int rc = alpha_moe_validate(top_k, M, K, N, num_experts, sorted_num, block_m, block_n, warp_n, stages);
+    if (rc != ALPHA_MOE_OK) return rc;
+    if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
+        workspace_bytes < alpha_moe_workspace_bytes(M, K, N, sorted_num, block_m))
+        return ALPHA_MOE_ERR_WORKSPACE;
+
+    MoeParams p;
+    p.x = x; p.x_scale = x_scale; p.w = w; p.w_scale = w_scale; p.w2 = w2; p.w2_scale = w2_scale;
+    p.out = out; p.acc = static_cast<float *>(workspace);
+    p.sorted_ids = sorted_token_ids; p.expert_ids = expert_ids; p.ntpp = num_tokens_post_padded;
+    p.topk_w = topk_weights;
+    p.top_k = top_k; p.M = M; p.K = K; p.N = N; p.E = num_experts; p.sorted_num = sorted_num; p.block_m = block_m;
+    p.scaling = scaling_factor;
+
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    hipError_t err;
+    if (use_stream(block_m)) {
+        err = launch_stream(p, warp_n, stages, workspace, hs);
+    } else {
+        err = launch_direct(p, warp_n, stages, hs);
+        if (err == hipSuccess) err = launch_finalize(p, hs);
+    }
+    return err == hipSuccess ? ALPHA_MOE_OK : ALPHA_MOE_ERR_LAUNCH;
+}
+
+extern "C" const char *alpha_moe_status_string(int status)
+{
+    switch (status) {
+    case ALPHA_MOE_OK: return "ok";
+    case ALPHA_MOE_ERR_NULL_POINTER: return "a required pointer is null";
+    case ALPHA_MOE_ERR_SHAPE: return "unsupported shape: need M>0, top_k>0, K % 128 == 0, K <= 65536, N % 256 == 0, sizes within int32";
+    case ALPHA_MOE_ERR_BLOCK_M: return "block_m must be a multiple of 8 in [8, 128]";
+    case ALPHA_MOE_ERR_BLOCK_N_WARP_N: return "(block_n, warp_n) must be (64, 4) or (32, 8)";
+    case ALPHA_MOE_ERR_STAGES: return "stages must be in [1, 5]";
+    case ALPHA_MOE_ERR_WORKSPACE: return "workspace is null, not 256-byte aligned, or smaller than alpha_moe_workspace_bytes()";
+    case ALPHA_MOE_ERR_LAUNCH: return "the HIP runtime refused the kernel launch";
+    default: return "unknown status";
+    }
+}
+
+extern "C" const char *alpha_moe_version(void) { return "0.2"; }

@@ -1,0 +1,111 @@
+// Shared device helpers and launch interfaces of the gfx950 fused W8A8 MoE kernels.
+//
+// Conventions used by every kernel in this directory:
+//   * v_mfma_f32_16x16x128_f8f6f4 with WEIGHT rows as the A operand and TOKENS as the B operand; one instruction
+//     contracts exactly one 128-wide scale block, so block scales multiply its fp32 result.
+//   * Operand lane layout: lane = (m = lane % 16, q = lane / 16); the lane feeds row/column m with the 32 bytes
+//     [16q, 16q+16) ++ [64+16q, 64+16q+16) of the 128-byte K block ("chunk q" and "chunk q+4" of eight 16-byte
+//     chunks).  Any K permutation is legal as long as A and B use the same one.
+//   * Accumulator lane layout: register j of lane (n, q) is (row 4q + j, token n).
+//   * Gate/up pairing under the interleave-8 weight layout: the gate MFMA of a 32-row group takes the 8+8 gate rows
+//     of its two 16-row chunks, the up MFMA their up rows, so accumulator j of a lane is gate/up of the SAME
+//     intermediate column and a lane owns 4 consecutive columns.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/alpha_moe_hip.h"
+
+namespace alpha_moe {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr float kFp8Max = 448.0f;
+constexpr float kAmaxFloor = 1e-10f;
+constexpr int kMaxKBlocks = 512;     // K <= 65536
+constexpr int kLdsRowStride = 144;   // 128 FP8 + 16 pad: dword writes of 16 tokens x 4 quads hit 64 distinct banks
+
+struct MoeParams {
+    const uint8_t *x;
+    const float *x_scale;
+    const uint8_t *w;
+    const float *w_scale;
+    const uint8_t *w2;
+    const float *w2_scale;
+    uint16_t *out;              // [M, K] bf16
+    float *acc;                 // [M, K] fp32 scratch, zero on entry, zero on exit
+    const int32_t *sorted_ids;
+    const int32_t *expert_ids;
+    const int32_t *ntpp;
+    const float *topk_w;
+    int top_k, M, K, N, E, sorted_num, block_m;
+    float scaling;
+};
+
+__device__ __forceinline__ v4i ldg128(const uint8_t *p) { return *reinterpret_cast<const v4i *>(p); }
+
+__device__ __forceinline__ v8i cat(v4i lo, v4i hi)
+{
+    return (v8i){lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+}
+
+__device__ __forceinline__ v4f mfma_fp8(v8i a, v8i b)
+{
+    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+    // cbsz = blgp = 0: both operands OCP e4m3; scale operands 0 -> plain v_mfma_f32_16x16x128_f8f6f4
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, zero, 0, 0, 0, 0, 0, 0);
+}
+
+__device__ __forceinline__ float round_bf16(float v) { return static_cast<float>(static_cast<__bf16>(v)); }
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
+{
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    bf2 p = {static_cast<__bf16>(lo), static_cast<__bf16>(hi)};
+    return __builtin_bit_cast(uint32_t, p);
+}
+
+__device__ __forceinline__ float clamp_fp8(float v) { return fminf(fmaxf(v, -kFp8Max), kFp8Max); }
+
+__device__ __forceinline__ uint32_t pack_fp8x4(float a, float b, float c, float d)
+{
+    int p = 0;
+    p = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, p, false);   // RNE to OCP e4m3 on gfx950
+    p = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, p, true);
+    return static_cast<uint32_t>(p);
+}
+
+// SwiGLU on bf16-rounded gate/up, result rounded to bf16 (the reference keeps all three in bf16,
+// fused_moe_w8a8_up_down_acc.cu:76-79,919-946)
+__device__ __forceinline__ float swiglu_bf16(float gate, float up)
+{
+    const float g = round_bf16(gate);
+    const float u = round_bf16(up);
+    return round_bf16(g / (1.0f + __expf(-g)) * u);
+}
+
+__device__ __forceinline__ void atomic_add_f32(float *addr, float v)
+{
+    typedef float __attribute__((address_space(1))) * gptr;
+    __builtin_amdgcn_global_atomic_fadd_f32(reinterpret_cast<gptr>(reinterpret_cast<uintptr_t>(addr)), v);
+}
+
+// ---- host-side launchers, one per kernel family (each in its own translation unit) -------------------------
+
+// One workgroup per (block of block_m sorted rows, 128-column intermediate slice), weights HBM -> VGPR.
+// Any block_m in 8..128.  Needs p.acc (M*K floats, zeroed) and finishes with the finalize kernel.
+hipError_t launch_direct(const MoeParams &p, int warp_n, int stages, hipStream_t stream);
+
+// out = bf16(out + acc); acc = 0
+hipError_t launch_finalize(const MoeParams &p, hipStream_t stream);
+
+// Persistent work-queue kernel for block_m <= 32: split-K up items -> SwiGLU/requant -> column-slab down items
+// -> finalize, chained through counters in the workspace.  Weights HBM -> LDS with direct-to-LDS loads.
+bool stream_supported(int block_m);
+size_t stream_workspace_bytes(int M, int K, int N, int sorted_num, int block_m);
+hipError_t launch_stream(const MoeParams &p, int warp_n, int stages, void *workspace, hipStream_t stream);
+
+}  // namespace alpha_moe

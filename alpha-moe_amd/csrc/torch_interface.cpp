@@ -14,7 +14,28 @@
 
 #include "../../include/alpha_moe_hip.h"
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 namespace {
+
+// Scratch for the C ABI, one buffer per (device, stream): zero-filled when created, left zero-filled by every
+// call, so the steady state allocates and clears nothing (the first call on a stream does both: warm the
+// operator up once before capturing it into a HIP graph).
+at::Tensor workspace_for(const at::Device &dev, hipStream_t stream, size_t bytes)
+{
+    static std::mutex mu;
+    static std::map<std::pair<int, void *>, at::Tensor> cache;
+    std::lock_guard<std::mutex> lock(mu);
+    at::Tensor &slot = cache[{dev.index(), static_cast<void *>(stream)}];
+    if (!slot.defined() || static_cast<size_t>(slot.numel()) < bytes) {
+        size_t cap = 1 << 20;
+        while (cap < bytes) cap <<= 1;
+        slot = at::zeros({static_cast<int64_t>(cap)}, at::TensorOptions().dtype(at::kByte).device(dev));
+    }
+    return slot;
+}
 
 void check_tensor(const at::Tensor &t, const char *name, at::ScalarType dtype, const at::Device &dev)
 {
@@ -71,6 +92,10 @@ void fused_moe_w8a8_up_down(const at::Tensor &x, const at::Tensor &x_scale, cons
     const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(dev);
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
 
+    const size_t ws_bytes = alpha_moe_workspace_bytes(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N),
+                                                      static_cast<int>(sorted_num), static_cast<int>(block_m));
+    at::Tensor ws = workspace_for(dev, stream, ws_bytes);
+
     const int rc = alpha_moe_fused_moe_w8a8_up_down(
         static_cast<const uint8_t *>(x.const_data_ptr()), x_scale.const_data_ptr<float>(),
         static_cast<const uint8_t *>(w.const_data_ptr()), w_scale.const_data_ptr<float>(),
@@ -80,7 +105,8 @@ void fused_moe_w8a8_up_down(const at::Tensor &x, const at::Tensor &x_scale, cons
         topk_weights.const_data_ptr<float>(), static_cast<int>(top_k), static_cast<int>(M), static_cast<int>(K),
         static_cast<int>(N), static_cast<int>(E), static_cast<int>(sorted_num), static_cast<int>(block_m),
         static_cast<int>(block_n), static_cast<int>(warp_n), static_cast<int>(stages),
-        static_cast<float>(scaling_factor), static_cast<void *>(stream));
+        static_cast<float>(scaling_factor), ws.data_ptr(), static_cast<size_t>(ws.numel()),
+        static_cast<void *>(stream));
     TORCH_CHECK(rc == ALPHA_MOE_OK, "alpha_moe_fused_moe_w8a8_up_down failed: ", alpha_moe_status_string(rc));
 }
 

@@ -8,6 +8,7 @@
 #ifndef ALPHA_MOE_HIP_H
 #define ALPHA_MOE_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -21,7 +22,8 @@ enum alpha_moe_status {
     ALPHA_MOE_ERR_BLOCK_M = 3,        /* block_m not in {8,16,...,128} */
     ALPHA_MOE_ERR_BLOCK_N_WARP_N = 4, /* (block_n, warp_n) not (64,4) or (32,8) */
     ALPHA_MOE_ERR_STAGES = 5,         /* stages not in 1..5 */
-    ALPHA_MOE_ERR_LAUNCH = 6          /* the HIP runtime refused the launch (see hipGetLastError) */
+    ALPHA_MOE_ERR_LAUNCH = 6,         /* the HIP runtime refused the launch (see hipGetLastError) */
+    ALPHA_MOE_ERR_WORKSPACE = 7       /* workspace null, misaligned or smaller than alpha_moe_workspace_bytes() */
 };
 
 /*
@@ -30,8 +32,9 @@ enum alpha_moe_status {
  * Replaces the reference's C++ seam `fused_moe_w8a8_wgmma_up_down_acc`
  * (declared csrc/torch_interface.cpp:12-34, defined
  * csrc/kernels/fused_moe_w8a8/fused_moe_w8a8_up_down_acc.cu:1258-1303): same parameters in the same order, with
- * fp8 as uint8_t codes (OCP e4m3fn), bf16 as uint16_t, the stream as an opaque hipStream_t, and an int status
- * instead of stderr prints / exit().
+ * fp8 as uint8_t codes (OCP e4m3fn), bf16 as uint16_t, the stream as an opaque hipStream_t, an int status
+ * instead of stderr prints / exit(), and a caller-owned scratch buffer before the stream (the reference has none:
+ * it adds every partial row straight into the bf16 output).
  *
  *   x                [M, K]            fp8, row-major, K % 128 == 0
  *   x_scale          [M, K/128]        f32, per token per 128 columns
@@ -39,7 +42,7 @@ enum alpha_moe_status {
  *   w_scale          [E, N/128, K/128] f32, gate/up rows interleaved in chunks of 1
  *   w2               [E, K, N/2]       fp8
  *   w2_scale         [E, K/128, N/256] f32
- *   out              [M, K]            bf16, the result is ADDED (packed bf16 atomics); caller zero-fills
+ *   out              [M, K]            bf16, the result is ADDED once per call (out = bf16(out + sum)); caller zero-fills
  *   sorted_token_ids [sorted_num]      flat slot ids t*top_k+s grouped by expert in blocks of block_m; ids >= M*top_k are padding
  *   expert_ids       [ceil(sorted_num/block_m)]  expert of each block (blocks with an id outside [0,E) are skipped)
  *   num_tokens_post_padded [1]         blocks starting at or past this row are skipped
@@ -47,6 +50,10 @@ enum alpha_moe_status {
  *   block_m          8..128 step 8     must equal the block size sorted_token_ids was built with
  *   (block_n, warp_n) (64,4) or (32,8) wavefronts per workgroup = warp_n, w1 rows per wavefront = block_n
  *   stages           1..5              K-blocks of loads kept in flight per wavefront
+ *   workspace        device scratch of at least alpha_moe_workspace_bytes(M, K, N, sorted_num, block_m) bytes,
+ *                    256-byte aligned.  It must be ZERO-FILLED before its first use; every call leaves it zero-filled
+ *                    again, so one buffer can be kept for the life of the process and serve calls of any sizes it is
+ *                    large enough for.  Calls that share a workspace must be ordered on one stream.
  */
 int alpha_moe_fused_moe_w8a8_up_down(
     const uint8_t *x, const float *x_scale,
@@ -57,7 +64,10 @@ int alpha_moe_fused_moe_w8a8_up_down(
     const float *topk_weights,
     int top_k, int M, int K, int N, int num_experts, int sorted_num,
     int block_m, int block_n, int warp_n, int stages,
-    float scaling_factor, void *stream /* hipStream_t */);
+    float scaling_factor, void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
+
+/* Bytes of scratch the call above needs for these sizes (0 if any is not positive). */
+size_t alpha_moe_workspace_bytes(int M, int K, int N, int sorted_num, int block_m);
 
 /*
  * The argument checks of the call above without touching the device: returns the status the launch would

@@ -28,6 +28,18 @@ def test_c1_default_knobs_torch_op_and_c_abi(c1):
     assert_parity(run_op(P, 16, 64, 4, 3, via="c_abi"), ref, "c abi")
 
 
+def test_c_abi_workspace_is_reusable_without_clearing(c1):
+    """One zero-filled workspace, many calls with different knobs (and so different kernels and layouts inside it)."""
+    import alpha_moe
+    P, ref = c1
+    sizes = [alpha_moe.c_abi.alpha_moe_workspace_bytes(P.M, P.shape.K, P.shape.N, P.align(bm)[0].numel(), bm)
+             for bm in (8, 16, 32, 64)]
+    ws = torch.zeros(max(sizes), dtype=torch.uint8, device=DEV)
+    for bm, bn, wn, st in [(16, 64, 4, 2), (16, 64, 4, 2), (8, 32, 8, 3), (64, 64, 4, 2), (32, 32, 8, 1), (16, 64, 4, 4)]:
+        print(f"case c1 shared workspace knobs {(bm, bn, wn, st)}", flush=True)
+        assert_parity(run_op(P, bm, bn, wn, st, via="c_abi", workspace=ws), ref, f"shared ws {(bm, bn, wn, st)}")
+
+
 def test_c1_result_independent_of_every_knob(c1):
     """The reference's correctness sweep runs every (block_m, block_n/warp_n, stages) it accepts
     (test_moe_correctness.py:172-190); the result may not depend on them."""
