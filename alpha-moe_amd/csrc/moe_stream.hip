@@ -87,6 +87,29 @@ __device__ __forceinline__ float ldg32_untracked(const float *p)
     return r;
 }
 
+// Agent-scope (sc1) accesses for data that crosses workgroups inside one launch: they are served at the point
+// where all XCDs agree, so no L2-wide write-back / invalidate (what a __threadfence() costs here) is needed.
+__device__ __forceinline__ v4i ldg128_agent(const void *p)
+{
+    v4i r;
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(r) : "v"(p) : "memory");
+    return r;
+}
+__device__ __forceinline__ void stg32_agent(void *p, uint32_t v)
+{
+    asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void stg128_agent(void *p, v4i v)
+{
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void atomic_add_f32_agent(float *p, float v)
+{
+    asm volatile("global_atomic_add_f32 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+// all of this wavefront's vector-memory operations (loads, stores, atomics) have completed
+__device__ __forceinline__ void drain_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt()
 {
@@ -245,13 +268,14 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                     pack_fp8x4(clamp_fp8(accg[pr][t][0] / s_a), clamp_fp8(accg[pr][t][1] / s_a),
                                clamp_fp8(accg[pr][t][2] / s_a), clamp_fp8(accg[pr][t][3] / s_a));
                 const int col = wave * (RW / 2) + pr * 16 + 4 * q;
-                *reinterpret_cast<uint32_t *>(aq_u + (t * 16 + n) * 128 + col) = packed;
+                stg32_agent(aq_u + (t * 16 + n) * 128 + col, packed);
             }
-            if (wave == 0 && q == 0) s.sa[(size_t)u * s.bm_pad + t * 16 + n] = s_a;
+            if (wave == 0 && q == 0)
+                stg32_agent(&s.sa[(size_t)u * s.bm_pad + t * 16 + n], __builtin_bit_cast(uint32_t, s_a));
         }
-        __threadfence();
+        drain_vmem();
         __syncthreads();
-        if (tid == 0) __hip_atomic_store(&s.flag[u], 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) store_agent(&s.flag[u], 1);
     };
 
     auto up_item = [&](int item) {
@@ -355,31 +379,33 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                     float *dst = h_u + (t * 16 + n) * 256 + wave * (RW / 2) + pr * 16 + 4 * q;
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
-                        atomic_add_f32(dst + j, accg[pr][t][j]);
-                        atomic_add_f32(dst + 128 + j, accu[pr][t][j]);
+                        atomic_add_f32_agent(dst + j, accg[pr][t][j]);
+                        atomic_add_f32_agent(dst + 128 + j, accu[pr][t][j]);
                     }
                 }
             }
-            __threadfence();
+            drain_vmem();
             __syncthreads();
             if (tid == 0)
-                s_bcast[1] = __hip_atomic_fetch_add(&s.arrive[u], 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+                s_bcast[1] = __hip_atomic_fetch_add(&s.arrive[u], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __syncthreads();
             if (s_bcast[1] != s.ks - 1) return;
-            __threadfence();
 #pragma unroll
             for (int t = 0; t < TM; t++)
 #pragma unroll
                 for (int pr = 0; pr < NP; pr++) {
-                    v4f *src = reinterpret_cast<v4f *>(h_u + (t * 16 + n) * 256 + wave * (RW / 2) + pr * 16 + 4 * q);
-                    const v4f zero = {0.f, 0.f, 0.f, 0.f};
-                    accg[pr][t] = zero;
-                    accu[pr][t] = zero;
+                    float *src = h_u + (t * 16 + n) * 256 + wave * (RW / 2) + pr * 16 + 4 * q;
+                    v4i g = {0, 0, 0, 0}, up = {0, 0, 0, 0};
                     if (r.valid[t]) {
-                        accg[pr][t] = src[0];
-                        accu[pr][t] = src[32];
-                        src[0] = zero;
-                        src[32] = zero;
+                        g = ldg128_agent(src);
+                        up = ldg128_agent(src + 128);
+                    }
+                    drain_vmem();
+                    accg[pr][t] = __builtin_bit_cast(v4f, g);
+                    accu[pr][t] = __builtin_bit_cast(v4f, up);
+                    if (r.valid[t]) {
+                        stg128_agent(src, (v4i){0, 0, 0, 0});
+                        stg128_agent(src + 128, (v4i){0, 0, 0, 0});
                     }
                 }
             if (tid == 0) store_agent(&s.arrive[u], 0);
@@ -396,7 +422,6 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         if (e >= 0 && e < p.E) {
             if (tid == 0) spin_until_ge(&s.flag[u], 1, s.ctl);
             __syncthreads();
-            __threadfence();
             const Routing<TM> r = load_routing<TM>(p, mb, n);
 
             const int t0 = cs * s.tpi;
@@ -417,8 +442,12 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             const uint8_t *aq_u = s.aq + (size_t)u * s.bm_pad * 128;
 #pragma unroll
             for (int t = 0; t < TM; t++) {
-                ba[t] = cat(ldg128(aq_u + (t * 16 + n) * 128 + 16 * q), ldg128(aq_u + (t * 16 + n) * 128 + 64 + 16 * q));
-                tsc[t] = s.sa[(size_t)u * s.bm_pad + t * 16 + n] * (p.topk_w[r.slot[t]] * p.scaling);
+                const v4i lo = ldg128_agent(aq_u + (t * 16 + n) * 128 + 16 * q);
+                const v4i hi = ldg128_agent(aq_u + (t * 16 + n) * 128 + 64 + 16 * q);
+                const int sa_bits = load_agent(reinterpret_cast<const int *>(&s.sa[(size_t)u * s.bm_pad + t * 16 + n]));
+                drain_vmem();
+                ba[t] = cat(lo, hi);
+                tsc[t] = __builtin_bit_cast(float, sa_bits) * (p.topk_w[r.slot[t]] * p.scaling);
                 accp[t] = p.acc + (size_t)r.tok[t] * K + 4 * q;
             }
             if (wnt > 0) {
@@ -454,7 +483,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                                 const float sc = tsc[t] * ws;
                                 if (r.valid[t]) {
 #pragma unroll
-                                    for (int jj = 0; jj < 4; jj++) atomic_add_f32(accp[t] + c0 + jj, d[jj] * sc);
+                                    for (int jj = 0; jj < 4; jj++) atomic_add_f32_agent(accp[t] + c0 + jj, d[jj] * sc);
                                 }
                             }
                         }
@@ -463,23 +492,24 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 pipeline<STAGES, LPS>(n_st, issue, compute);
             }
         }
-        __threadfence();
+        drain_vmem();
         __syncthreads();
-        if (tid == 0) __hip_atomic_fetch_add(&s.ctl->down_done, 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) __hip_atomic_fetch_add(&s.ctl->down_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
 
     auto fin_item = [&](int f) {
         if (tid == 0) spin_until_ge(&s.ctl->down_done, n_down, s.ctl);
         __syncthreads();
-        __threadfence();
         const int n4 = (int)(((int64_t)p.M * K) >> 2);
         const int i = f * FIN_CHUNK + tid;
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             const int idx = i + k * THREADS;
             if (idx < n4) {
-                v4f a = reinterpret_cast<v4f *>(p.acc)[idx];
+                const v4i a_bits = ldg128_agent(reinterpret_cast<const v4f *>(p.acc) + idx);
                 uint2 o = reinterpret_cast<uint2 *>(p.out)[idx];
+                drain_vmem();
+                const v4f a = __builtin_bit_cast(v4f, a_bits);
                 const float o0 = __builtin_bit_cast(float, o.x << 16), o1 = __builtin_bit_cast(float, o.x & 0xffff0000u);
                 const float o2 = __builtin_bit_cast(float, o.y << 16), o3 = __builtin_bit_cast(float, o.y & 0xffff0000u);
                 o.x = pack_bf16x2(o0 + a[0], o1 + a[1]);
@@ -521,7 +551,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         item = s_bcast[0];
     }
     if (tid == 0) {
-        const int left = __hip_atomic_fetch_add(&s.ctl->done, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const int left = __hip_atomic_fetch_add(&s.ctl->done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (left == (int)gridDim.x - 1) {
             store_agent(&s.ctl->head, 0);
             store_agent(&s.ctl->done, 0);
