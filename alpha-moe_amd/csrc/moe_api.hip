@@ -21,9 +21,9 @@ int forced_path()
     return v;
 }
 
-bool use_stream(int block_m)
+bool use_stream(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
 {
-    if (!stream_supported(block_m)) return false;
+    if (!stream_supported(top_k, M, K, N, E, sorted_num, block_m)) return false;
     return forced_path() != 1;
 }
 
@@ -43,11 +43,16 @@ extern "C" int alpha_moe_validate(int top_k, int M, int K, int N, int num_expert
     return ALPHA_MOE_OK;
 }
 
-extern "C" size_t alpha_moe_workspace_bytes(int M, int K, int N, int sorted_num, int block_m)
+extern "C" size_t alpha_moe_workspace_bytes(int top_k, int M, int K, int N, int num_experts, int sorted_num,
+                                            int block_m)
 {
-    if (M <= 0 || K <= 0 || N <= 0 || sorted_num <= 0 || block_m <= 0) return 0;
-    const size_t direct = (size_t)M * (size_t)K * sizeof(float);
-    const size_t stream = stream_supported(block_m) ? stream_workspace_bytes(M, K, N, sorted_num, block_m) : 0;
+    if (top_k <= 0 || M <= 0 || K <= 0 || N <= 0 || num_experts <= 0 || sorted_num <= 0 || block_m <= 0) return 0;
+    // both kernel families keep their bookkeeping out of each other's way: the streaming kernel's self-maintaining
+    // prefix comes first, the direct kernel's accumulator (cleared on every call) after it
+    const size_t direct = stream_prefix_bytes() + (size_t)M * (size_t)K * sizeof(float);
+    const size_t stream = stream_supported(top_k, M, K, N, num_experts, sorted_num, block_m)
+                              ? stream_workspace_bytes(top_k, M, K, N, num_experts, sorted_num, block_m)
+                              : 0;
     return direct > stream ? direct : stream;
 }
 
@@ -66,12 +71,13 @@ extern "C" int alpha_moe_fused_moe_w8a8_up_down(const uint8_t *x, const float *x
     const int rc = alpha_moe_validate(top_k, M, K, N, num_experts, sorted_num, block_m, block_n, warp_n, stages);
     if (rc != ALPHA_MOE_OK) return rc;
     if (!workspace || (reinterpret_cast<uintptr_t>(workspace) & 255) != 0 ||
-        workspace_bytes < alpha_moe_workspace_bytes(M, K, N, sorted_num, block_m))
+        workspace_bytes < alpha_moe_workspace_bytes(top_k, M, K, N, num_experts, sorted_num, block_m))
         return ALPHA_MOE_ERR_WORKSPACE;
 
     MoeParams p;
     p.x = x; p.x_scale = x_scale; p.w = w; p.w_scale = w_scale; p.w2 = w2; p.w2_scale = w2_scale;
-    p.out = out; p.acc = static_cast<float *>(workspace);
+    p.out = out;
+    p.acc = reinterpret_cast<float *>(static_cast<uint8_t *>(workspace) + stream_prefix_bytes());
     p.sorted_ids = sorted_token_ids; p.expert_ids = expert_ids; p.ntpp = num_tokens_post_padded;
     p.topk_w = topk_weights;
     p.top_k = top_k; p.M = M; p.K = K; p.N = N; p.E = num_experts; p.sorted_num = sorted_num; p.block_m = block_m;
@@ -79,10 +85,11 @@ extern "C" int alpha_moe_fused_moe_w8a8_up_down(const uint8_t *x, const float *x
 
     hipStream_t hs = static_cast<hipStream_t>(stream);
     hipError_t err;
-    if (use_stream(block_m)) {
+    if (use_stream(top_k, M, K, N, num_experts, sorted_num, block_m)) {
         err = launch_stream(p, warp_n, stages, workspace, hs);
     } else {
-        err = launch_direct(p, warp_n, stages, hs);
+        err = launch_zero_acc(p, hs);
+        if (err == hipSuccess) err = launch_direct(p, warp_n, stages, hs);
         if (err == hipSuccess) err = launch_finalize(p, hs);
     }
     return err == hipSuccess ? ALPHA_MOE_OK : ALPHA_MOE_ERR_LAUNCH;

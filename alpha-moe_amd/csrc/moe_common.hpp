@@ -36,7 +36,7 @@ struct MoeParams {
     const uint8_t *w2;
     const float *w2_scale;
     uint16_t *out;              // [M, K] bf16
-    float *acc;                 // [M, K] fp32 scratch, zero on entry, zero on exit
+    float *acc;                 // [M, K] fp32 scratch (direct kernel only)
     const int32_t *sorted_ids;
     const int32_t *expert_ids;
     const int32_t *ntpp;
@@ -96,16 +96,18 @@ __device__ __forceinline__ void atomic_add_f32(float *addr, float v)
 // ---- host-side launchers, one per kernel family (each in its own translation unit) -------------------------
 
 // One workgroup per (block of block_m sorted rows, 128-column intermediate slice), weights HBM -> VGPR.
-// Any block_m in 8..128.  Needs p.acc (M*K floats, zeroed) and finishes with the finalize kernel.
+// Any block_m in 8..128.  Adds into p.acc (M*K floats, cleared by launch_zero_acc first); launch_finalize then
+// rounds the sums into p.out.
+hipError_t launch_zero_acc(const MoeParams &p, hipStream_t stream);
 hipError_t launch_direct(const MoeParams &p, int warp_n, int stages, hipStream_t stream);
+hipError_t launch_finalize(const MoeParams &p, hipStream_t stream);   // out = bf16(out + acc)
 
-// out = bf16(out + acc); acc = 0
-hipError_t launch_finalize(const MoeParams &p, hipStream_t stream);
-
-// Persistent work-queue kernel for block_m <= 32: split-K up items -> SwiGLU/requant -> column-slab down items
-// -> finalize, chained through counters in the workspace.  Weights HBM -> LDS with direct-to-LDS loads.
-bool stream_supported(int block_m);
-size_t stream_workspace_bytes(int M, int K, int N, int sorted_num, int block_m);
+// Persistent work-queue kernel for decode-sized batches (block_m <= 32 and bounded sizes): split-K up items ->
+// SwiGLU/requant -> column-slab down items -> per-token reduction, chained through counters in the workspace.
+// Weights HBM -> LDS with direct-to-LDS loads.  The first stream_prefix_bytes() of the workspace belong to it.
+size_t stream_prefix_bytes();
+bool stream_supported(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
+size_t stream_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
 hipError_t launch_stream(const MoeParams &p, int warp_n, int stages, void *workspace, hipStream_t stream);
 
 }  // namespace alpha_moe

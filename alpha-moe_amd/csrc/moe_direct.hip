@@ -7,8 +7,8 @@
 // Each wavefront owns its own weight rows, so nothing is shared between wavefronts until the 128-column
 // requantisation group is reduced; the requantised block_m x 128 FP8 tile crosses lanes once through LDS
 // (accumulator layout != B layout).  Down projection: w2 rows (= output columns) as A gives each lane 4 adjacent
-// output columns of one token.  Partial output rows are summed in an fp32 scratch row with hardware fp32 atomics
-// and rounded to bf16 once by the finalize kernel (adding every partial straight into the bf16 output would round
+// output columns of one token.  Partial output rows are summed in an fp32 scratch row (cleared by a fill kernel
+// first) with hardware fp32 atomics and rounded to bf16 once by the finalize kernel (adding every partial straight into the bf16 output would round
 // the running sum top_k * I/128 times, ~1.5e-2 of the output range for DeepSeek-V3 routing weights).
 //
 // Handles every block_m in 8..128; the persistent streaming kernel in moe_stream.hip is the fast path for
@@ -251,7 +251,13 @@ __global__ __launch_bounds__(WN * 64) void fused_moe_w8a8_direct_kernel(const Mo
     }
 }
 
-// out[i] = bf16(float(out[i]) + acc[i]); acc[i] = 0.  n4 = M*K/4 (K % 128 == 0, so rows never straddle).
+__global__ __launch_bounds__(256) void moe_zero_kernel(float *__restrict__ acc, int n4)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n4) reinterpret_cast<v4f *>(acc)[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+}
+
+// out[i] = bf16(float(out[i]) + acc[i]).  n4 = M*K/4 (K % 128 == 0, so rows never straddle).
 __global__ __launch_bounds__(256) void moe_finalize_kernel(float *__restrict__ acc, uint16_t *__restrict__ out, int n4)
 {
     const int i = blockIdx.x * 256 + threadIdx.x;
@@ -263,7 +269,6 @@ __global__ __launch_bounds__(256) void moe_finalize_kernel(float *__restrict__ a
     o.x = pack_bf16x2(o0 + a[0], o1 + a[1]);
     o.y = pack_bf16x2(o2 + a[2], o3 + a[3]);
     reinterpret_cast<uint2 *>(out)[i] = o;
-    reinterpret_cast<v4f *>(acc)[i] = (v4f){0.f, 0.f, 0.f, 0.f};
 }
 
 typedef void (*KernelFn)(const MoeParams);
@@ -314,6 +319,14 @@ hipError_t launch_direct(const MoeParams &p, int warp_n, int stages, hipStream_t
     const int n_blocks = (p.sorted_num + p.block_m - 1) / p.block_m;
     const dim3 grid((unsigned)(n_blocks * (p.N / 256)));
     hipLaunchKernelGGL(fn, grid, dim3((unsigned)(warp_n * 64)), 0, stream, p);
+    return hipGetLastError();
+}
+
+hipError_t launch_zero_acc(const MoeParams &p, hipStream_t stream)
+{
+    // a fill kernel, not hipMemsetAsync: the call may be captured into a HIP graph
+    const int n4 = (int)((int64_t)p.M * p.K / 4);
+    hipLaunchKernelGGL(moe_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, p.acc, n4);
     return hipGetLastError();
 }
 

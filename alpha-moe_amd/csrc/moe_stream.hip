@@ -7,26 +7,34 @@
 // engage all 256 CUs.  The 128-column requantisation group forces a dependency between the pieces, so the kernel
 // is a small dataflow over a work queue (items are taken in queue order with one atomic):
 //
-//   UP item   (unit u = (row block mb, slice ib), K split ks): 256 interleaved w1 rows x kbpi K blocks.  Partial
-//             gate/up sums of the VALID tokens are added into h[u] (fp32 atomics); the item that arrives last at
-//             arrive[u] reads h[u], applies SwiGLU, quantises the block_m x 128 tile to FP8 (aq[u], sa[u]) and
-//             publishes flag[u] = 1.  With a single K split the sums never leave registers.
-//   DOWN item (unit u, column slab cs): waits for flag[u], then tpi 16-column tiles of w2[e][:, 128*ib : +128];
-//             results are added into acc[token] (fp32 atomics), then down_done is bumped.
-//   FIN item  (chunk of acc): waits for down_done == number of DOWN items, then out = bf16(out + acc), acc = 0,
-//             and clears its share of flag/aq/sa.
+//   UP item   (unit u = (row block mb, slice ib), K split ks): 256 interleaved w1 rows x kbpi K blocks.  With one
+//             K split the gate/up sums stay in registers; otherwise the VALID tokens' partial sums are stored to
+//             hpart[u][ks] and the item that arrives last at arrive[u] adds the slices up in a fixed order.  That
+//             workgroup applies SwiGLU, quantises the block_m x 128 tile to FP8 (aq[u], sa[u]) and publishes
+//             flag[u] = epoch.
+//   DOWN item (row block mb, column slab cs): waits for the flags of all I/128 slices of mb, then contracts the
+//             full intermediate against tpi 16-column tiles of w2[e] and stores each valid (token, slot) row's
+//             fp32 result to y[slot] - every element of y has exactly one writer.  Bumps down_done.
+//   FIN item  (token t, 1024 output columns): waits for down_done == number of DOWN items, then
+//             out[t] = bf16(out[t] + sum over the token's live slots of y[slot]) - one rounding, fixed order.
+//
+// There is no floating-point atomic anywhere: the result is bit-reproducible from run to run.
 //
 // Every wait is on items EARLIER in the queue, which are already held by running workgroups that never wait on
 // later ones, so the queue drains whatever the number of resident workgroups; each spin is bounded and sets
-// ctl->error instead of hanging.  Everything in the workspace is zero again when the kernel ends (arrive, h and acc
-// are cleared by their last reader, flag/aq/sa by the FIN items, head/done/down_done by the last workgroup to
-// leave), so one zero-filled buffer serves calls of any size without a memset in between.
+// ctl->error instead of hanging.  The workspace starts zero-filled; its first kPrefixBytes hold the control block,
+// the arrival counters (reset by the last arrival) and epoch-stamped flags, so nothing has to be cleared between
+// launches; the rest (aq, sa, hpart, y) is only ever read after it was written in the same launch.
 //
-// Data movement: weights go HBM -> LDS with non-temporal global_load_lds_dwordx4 (measured: 6.9 TB/s against
-// 3.4 TB/s for the same loads without the non-temporal hint, and 5.5 TB/s for direct-to-VGPR loads in the MFMA
-// lane order), into a per-wavefront ring of 16-row x 128-byte tiles, so the loop needs no workgroup barrier.  Inside
-// a tile, 16-byte chunk c of row m sits at position c ^ ((m >> 1) & 7): the MFMA operand read (16 rows at a fixed
-// chunk) then touches 16 distinct bank quads.  Token rows (a few KB, L2-resident) are loaded straight to VGPRs.
+// Data movement: weights go HBM -> LDS with non-temporal global_load_lds_dwordx4 (measured on MI355X: 6.9 TB/s
+// against 3.4 TB/s for the same loads without the non-temporal hint, and 5.5 TB/s for direct-to-VGPR loads in the
+// MFMA lane order), into a per-wavefront ring of 2 KiB tiles (16 rows x 128 bytes), so the loops need no workgroup
+// barrier.  Inside a tile, 16-byte chunk c of row m sits at position c ^ ((m >> 1) & 7): the MFMA operand read (16
+// rows at a fixed chunk) then touches 16 distinct bank quads.  A tile is exactly two load instructions, so "tile j
+// has landed" is "at most 2*(S-1) vector-memory operations outstanding" once the S-1 tiles behind it are issued;
+// result stores issued in between only make that wait stricter, never wrong.
+// Data that crosses workgroups inside the launch uses agent-scope (sc1) loads and stores: an L2-wide write-back /
+// invalidate (__threadfence) per hand-over costs ~4x the whole kernel on this 8-XCD part.
 #include <stdlib.h>
 
 #include <mutex>
@@ -37,58 +45,57 @@
 namespace alpha_moe {
 namespace {
 
+constexpr int kItemKBlocks = 64;     // most K blocks one UP item covers
+constexpr int kMaxIb = 16;           // most 128-column slices of the intermediate (I <= 2048)
+constexpr int kMaxUnits = 1 << 16;   // most (row block, slice) units of one launch
+constexpr int kMaxSlots = 1 << 18;   // most (token, slot) rows of one launch
+constexpr int kFinCols = 1024;       // output columns per FIN item
+
 struct StreamCtl {
     int head;        // next work item
     int done;        // workgroups that have left
-    int reserved;
+    int epoch;       // completed launches on this workspace
     int down_done;   // finished DOWN items of this launch
     int error;       // sticky: a bounded wait ran out
     int pad[59];
 };
 static_assert(sizeof(StreamCtl) == 256, "control block is one 256-byte line group");
 
+// zero-initialised, self-maintaining part of the workspace; its size does not depend on the problem
+constexpr size_t kOffArrive = 256;
+constexpr size_t kOffFlag = kOffArrive + sizeof(int) * kMaxUnits;
+constexpr size_t kOffLive = kOffFlag + sizeof(int) * kMaxUnits;
+constexpr size_t kPrefixBytes = kOffLive + sizeof(int) * kMaxSlots;
+
 struct StreamPlan {
     MoeParams p;
     StreamCtl *ctl;
-    int *arrive;     // [units]
-    int *flag;       // [units]
-    float *sa;       // [units][bm_pad]           requantisation scale per token
-    uint8_t *aq;     // [units][bm_pad][128]      requantised SwiGLU output, FP8
-    float *h;        // [units][bm_pad][2][128]   partial gate/up sums (K-split only)
+    int *arrive;     // [units]  K-split items that have delivered their partial sums
+    int *flag;       // [units]  == epoch once aq/sa of the unit are published
+    int *live;       // [slots]  == epoch once y[slot] is being written this launch
+    float *sa;       // [units][bm_pad]              requantisation scale per token
+    uint8_t *aq;     // [units][bm_pad][128]         requantised SwiGLU output, FP8
+    float *hpart;    // [units][ks][bm_pad][2][128]  partial gate/up sums (K-split only)
+    float *y;        // [slots][K]                   down-projection result per (token, slot) row
     int n_ib, nkb, n_ct, n_mb_max;
     int kbpi, ks;    // K blocks per UP item, UP items per unit
-    int tpi, n_cs;   // 16-column tiles per DOWN item, DOWN items per unit
-    int n_fin;       // FIN items
+    int tpi, n_cs;   // 16-column tiles per DOWN item, DOWN items per row block
+    int n_fc;        // FIN items per token
     int bm_pad;
 };
 
 typedef const void __attribute__((address_space(1))) * gptr_t;
 typedef void __attribute__((address_space(3))) * lptr_t;
 
-// 64 lanes x 16 bytes, HBM -> LDS at lds + lane*16, bypassing VGPRs; aux 2 = non-temporal
-__device__ __forceinline__ void dma16_nt(const uint8_t *g, uint8_t *lds)
+// 64 lanes x 16 bytes, memory -> LDS at lds + lane*16, bypassing VGPRs.  AUX: 0 default, 2 non-temporal, 16 agent scope
+template <int AUX>
+__device__ __forceinline__ void dma16(const uint8_t *g, uint8_t *lds)
 {
-    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uint32_t)(uintptr_t)lds, 16, 0, 2);
+    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uint32_t)(uintptr_t)lds, 16, 0, AUX);
 }
 
-// Global loads the compiler does not track: the pipelines below count vector-memory operations themselves and
-// place their own s_waitcnt vmcnt(N) (the compiler cannot see direct-to-LDS loads complete and, left to insert the
-// waits for ordinary loads mixed in between them, drains the whole queue every iteration).
-__device__ __forceinline__ v4i ldg128_untracked(const uint8_t *p, int byte_offset)
-{
-    v4i r;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r) : "v"(p + byte_offset) : "memory");
-    return r;
-}
-__device__ __forceinline__ float ldg32_untracked(const float *p)
-{
-    float r;
-    asm volatile("global_load_dword %0, %1, off" : "=v"(r) : "v"(p) : "memory");
-    return r;
-}
-
-// Agent-scope (sc1) accesses for data that crosses workgroups inside one launch: they are served at the point
-// where all XCDs agree, so no L2-wide write-back / invalidate (what a __threadfence() costs here) is needed.
+// Agent-scope (sc1) accesses for data that crosses workgroups inside one launch.  The loads are invisible to the
+// compiler's wait-count insertion: drain_vmem() before using their results.
 __device__ __forceinline__ v4i ldg128_agent(const void *p)
 {
     v4i r;
@@ -99,52 +106,26 @@ __device__ __forceinline__ void stg32_agent(void *p, uint32_t v)
 {
     asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
 }
-__device__ __forceinline__ void stg128_agent(void *p, v4i v)
+__device__ __forceinline__ void stg128_agent(void *p, v4f v)
 {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    // The hardware reads the data registers of a store wider than 64 bits a few cycles after issue; the compiler's
+    // hazard recognizer cannot see into inline asm, so the wait states before those registers may be overwritten
+    // are spelled out here.
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" ::"v"(p), "v"(v) : "memory");
 }
-__device__ __forceinline__ void atomic_add_f32_agent(float *p, float v)
+// all of this wavefront's vector-memory operations (loads, stores, direct-to-LDS loads) have completed
+__device__ __forceinline__ void drain_vmem()
 {
-    asm volatile("global_atomic_add_f32 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
 }
-// all of this wavefront's vector-memory operations (loads, stores, atomics) have completed
-__device__ __forceinline__ void drain_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 template <int N>
 __device__ __forceinline__ void wait_vmcnt()
 {
     static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-    __builtin_amdgcn_sched_barrier(0);   // consumers of untracked loads must not be scheduled above the wait
-}
-
-// STAGES-deep software pipeline over n steps.  issue(slot, step) must clamp `step` itself (prefetches past the end
-// are issued unconditionally so that the steady-state loop is branch-free) and issues exactly LPS vector-memory
-// instructions; compute(slot, step) consumes them.
-template <int STAGES, int LPS, class Issue, class Compute>
-__device__ __forceinline__ void pipeline(int n, Issue issue, Compute compute)
-{
-#pragma unroll
-    for (int s = 0; s < STAGES - 1; s++) issue(s, s);
-    const int n_full = n - n % STAGES;
-    for (int i0 = 0; i0 < n_full; i0 += STAGES) {
-#pragma unroll
-        for (int s = 0; s < STAGES; s++) {
-            issue((s + STAGES - 1) % STAGES, i0 + s + STAGES - 1);
-            __builtin_amdgcn_sched_barrier(0);
-            wait_vmcnt<(STAGES - 1) * LPS>();
-            compute(s, i0 + s);
-            __builtin_amdgcn_sched_barrier(0);
-        }
-    }
-    if constexpr (STAGES > 1) {
-        // drain: slots 0..STAGES-2 are in flight, oldest first.  Waiting for all of them at once costs nothing here.
-        wait_vmcnt<0>();
-#pragma unroll
-        for (int s = 0; s < STAGES - 1; s++)
-            if (n_full + s < n) compute(s, n_full + s);
-    }
-    wait_vmcnt<0>();
+    __builtin_amdgcn_sched_barrier(0);   // nothing that consumes the awaited data may be scheduled above the wait
 }
 
 __device__ __forceinline__ int load_agent(const int *p)
@@ -165,6 +146,30 @@ __device__ __noinline__ void spin_until_ge(const int *addr, int target, StreamCt
     }
     store_agent(&ctl->error, 1);
 }
+
+#ifdef ALPHA_MOE_TRACE
+// Debug builds only: per-item timestamps (100 MHz wall clock) for timeline analysis.
+__device__ unsigned long long g_trace[1 << 16][4];
+__device__ int g_trace_n;
+#define TRACE_VARS unsigned long long tr_t0 = 0, tr_t1 = 0
+#define TRACE_BEGIN tr_t0 = tr_t1 = wall_clock64()
+#define TRACE_MARK tr_t1 = wall_clock64()
+#define TRACE_END(kind, idx)                                                                        \
+    if (threadIdx.x == 0) {                                                                         \
+        const int slot_ = atomicAdd(&g_trace_n, 1);                                                 \
+        if (slot_ < (1 << 16)) {                                                                    \
+            g_trace[slot_][0] = ((unsigned long long)(kind) << 56) | ((unsigned long long)blockIdx.x << 32) | (unsigned)(idx); \
+            g_trace[slot_][1] = tr_t0;                                                              \
+            g_trace[slot_][2] = tr_t1;                                                              \
+            g_trace[slot_][3] = wall_clock64();                                                     \
+        }                                                                                           \
+    }
+#else
+#define TRACE_VARS
+#define TRACE_BEGIN
+#define TRACE_MARK
+#define TRACE_END(kind, idx)
+#endif
 
 template <int TM>
 struct Routing {
@@ -191,30 +196,35 @@ __device__ __forceinline__ Routing<TM> load_routing(const MoeParams &p, int mb, 
     return r;
 }
 
-template <int TM, int WN, int STAGES>
+// TM: 16-token tiles per row block; WN: wavefronts per workgroup; S: 2 KiB tiles in each wavefront's LDS ring
+template <int TM, int WN, int S>
 __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
 {
     constexpr int RW = 256 / WN;            // w1 rows per wavefront
     constexpr int NP = RW / 32;             // gate/up MFMA pairs per wavefront per K block
-    constexpr int NT = 2 * NP;              // 16x128 weight tiles per wavefront per UP stage
-    constexpr int DT = RW / 16;             // 16x128 weight tiles per wavefront per DOWN stage
-    constexpr int STAGE_BYTES = RW * 128;
+    constexpr int NT = 2 * NP;              // 16x128 weight tiles per wavefront per K block
+    constexpr int TPK = NT + TM;            // ring tiles per wavefront per K block (token tiles first)
     constexpr int THREADS = WN * 64;
-    constexpr int FIN_CHUNK = THREADS * 4;  // float4 elements per FIN item
+    static_assert(S >= 2 && 2 * (S - 1) < 64, "ring depth must fit the 6-bit vmcnt");
 
-    extern __shared__ __attribute__((aligned(1024))) uint8_t ring_all[];
-    __shared__ float s_ws[2][kMaxKBlocks];
+    // dynamic LDS: [WN rings of S tiles][n_ib * TM tiles of requantised activations (DOWN items)]
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds_dyn[];
+    __shared__ float s_sc[1024];                       // UP: gate scales [0,64), up scales [64,128); DOWN: w2 scales [blk][ib]
+    __shared__ float s_xs[TM * 16][kItemKBlocks + 1];  // UP: activation scales [row][K block]; DOWN: sa [row][ib]
+    __shared__ int s_tok[TM * 16];
     __shared__ float s_amax[WN][TM * 16];
     __shared__ int s_bcast[2];
 
+    TRACE_VARS;
     const MoeParams &p = s.p;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform, and the compiler should know it
     const int n = lane & 15;
     const int q = lane >> 4;
     const int K = p.K, I = p.N >> 1;
-    uint8_t *ring = ring_all + wave * (STAGES * STAGE_BYTES);
+    uint8_t *ring = lds_dyn + wave * (S * 2048);
+    uint8_t *s_aq = lds_dyn + WN * (S * 2048);
 
     // operand read offsets inside a 16x128 tile (see the swizzle note at the top of the file)
     const int f_n = (n >> 1) & 7;
@@ -226,12 +236,15 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
 #pragma unroll
     for (int i = 0; i < 2; i++) ld_chunk[i] = (lane & 7) ^ (((8 * i + ld_row) >> 1) & 7);
 
-    int n_mb = (s.p.ntpp[0] + p.block_m - 1) / p.block_m;
+    int n_mb = (__builtin_amdgcn_readfirstlane(s.p.ntpp[0]) + p.block_m - 1) / p.block_m;
     n_mb = n_mb < s.n_mb_max ? n_mb : s.n_mb_max;
     const int n_units = n_mb * s.n_ib;
     const int n_up = n_units * s.ks;
-    const int n_down = n_units * s.n_cs;
-    const int total = n_up + n_down + s.n_fin;
+    const int n_down = n_mb * s.n_cs;
+    const int n_fin = p.M * s.n_fc;
+    const int total = n_up + n_down + n_fin;
+    const int epoch = __builtin_amdgcn_readfirstlane(s.ctl->epoch) + 1;
+    const uint8_t *dummy = p.x;   // where loads past the end of an item are pointed: always mapped, always cached
 
     auto read_tile = [&](const uint8_t *tile) -> v8i {
         return cat(*reinterpret_cast<const v4i *>(tile + frag_lo), *reinterpret_cast<const v4i *>(tile + frag_hi));
@@ -275,7 +288,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         }
         drain_vmem();
         __syncthreads();
-        if (tid == 0) store_agent(&s.flag[u], 1);
+        if (tid == 0) store_agent(&s.flag[u], epoch);
     };
 
     auto up_item = [&](int item) {
@@ -283,38 +296,50 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         const int ksp = item - u * s.ks;
         const int mb = u / s.n_ib;
         const int ib = u - mb * s.n_ib;
-        const int e = p.expert_ids[mb];
+        const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
         if (e < 0 || e >= p.E) return;
         const int kb0 = ksp * s.kbpi;
         const int nk = (s.nkb - kb0) < s.kbpi ? (s.nkb - kb0) : s.kbpi;
         const Routing<TM> r = load_routing<TM>(p, mb, n);
 
-        // this unit's gate (row 2*ib) and up (row 2*ib+1) scale rows, K range of the item
+        // per-item tables in LDS: token of every row, the unit's gate (row 2*ib) / up (row 2*ib+1) weight scales and
+        // the tokens' activation scales over the item's K range
+        if (tid < TM * 16) {
+            const int idx = mb * p.block_m + tid;
+            int id = -1;
+            if (tid < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
+            const int tk = id / p.top_k;
+            s_tok[tid] = (id >= 0 && tk < p.M) ? tk : 0;
+        }
         {
             const float *ws_rows = p.w_scale + ((size_t)e * (p.N >> 7) + 2 * ib) * s.nkb + kb0;
             for (int i = tid; i < 2 * nk; i += THREADS) {
                 const int up = i >= nk;
-                s_ws[up][i - up * nk] = ws_rows[up * s.nkb + (i - up * nk)];
+                s_sc[up * kItemKBlocks + i - up * nk] = ws_rows[up * s.nkb + (i - up * nk)];
             }
         }
         __syncthreads();
+        for (int i = tid; i < TM * 16 * nk; i += THREADS) {
+            const int row = i / nk, k = i - row * nk;
+            s_xs[row][k] = p.x_scale[(size_t)s_tok[row] * s.nkb + kb0 + k];
+        }
 
+        // loader-side row pointers: tile position (row 8i + l/8, chunk slot l%8) <- global (row, chunk slot ^ f(row))
         const uint8_t *ga[NT][2];
 #pragma unroll
         for (int a = 0; a < NT; a++)
 #pragma unroll
             for (int i = 0; i < 2; i++) {
-                // tile a = (pair a/2, gate|up a%2); tile row 8i + l/8 is slab row pair*32 + 16i + l/8 (+8 for up)
+                // weight tile a = (pair a/2, gate|up a%2): tile row 8i + l/8 is slab row pair*32 + 16i + l/8 (+8 for up)
                 const int row = ib * 256 + wave * RW + (a >> 1) * 32 + 16 * i + ld_row + 8 * (a & 1);
                 ga[a][i] = p.w + ((size_t)e * p.N + row) * K + (size_t)kb0 * 128 + 16 * ld_chunk[i];
             }
-        const uint8_t *xp[TM];
-        const float *xsp[TM];
+        const uint8_t *gb[TM][2];
 #pragma unroll
-        for (int t = 0; t < TM; t++) {
-            xp[t] = p.x + (size_t)r.tok[t] * K + (size_t)kb0 * 128 + 16 * q;
-            xsp[t] = p.x_scale + (size_t)r.tok[t] * s.nkb + kb0;
-        }
+        for (int t = 0; t < TM; t++)
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                gb[t][i] = p.x + (size_t)s_tok[t * 16 + 8 * i + ld_row] * K + (size_t)kb0 * 128 + 16 * ld_chunk[i];
 
         v4f accg[NP][TM], accu[NP][TM];
 #pragma unroll
@@ -325,63 +350,74 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 accu[pr][t] = (v4f){0.f, 0.f, 0.f, 0.f};
             }
 
-        struct BStage {
-            v4i b[TM][2];
-            float xs[TM];
-        } bst[STAGES];
-        constexpr int LPS = NT * 2 + TM * 3;
-
-        auto issue = [&](int slot, int kb) {
-            kb = kb < nk ? kb : nk - 1;
-            uint8_t *dst = ring + slot * STAGE_BYTES;
+        // Tile stream of this wavefront: K block kb contributes TPK tiles in the order [tokens t=0..TM-1, G0, U0, G1, ...].
+        auto issue = [&](int kb, int a, int slot) {   // `a` is a compile-time constant after unrolling
+            uint8_t *dst = ring + slot * 2048;
+            const bool past_end = kb >= nk;
 #pragma unroll
-            for (int a = 0; a < NT; a++)
-#pragma unroll
-                for (int i = 0; i < 2; i++) dma16_nt(ga[a][i] + (size_t)kb * 128, dst + a * 2048 + i * 1024);
-#pragma unroll
-            for (int t = 0; t < TM; t++) {
-                bst[slot].b[t][0] = ldg128_untracked(xp[t] + (size_t)kb * 128, 0);
-                bst[slot].b[t][1] = ldg128_untracked(xp[t] + (size_t)kb * 128, 64);
-                bst[slot].xs[t] = ldg32_untracked(xsp[t] + kb);
+            for (int i = 0; i < 2; i++) {
+                if (a < TM)
+                    dma16<0>(past_end ? dummy : gb[a < TM ? a : 0][i] + (size_t)kb * 128, dst + i * 1024);
+                else
+                    dma16<2>(past_end ? dummy : ga[a >= TM ? a - TM : 0][i] + (size_t)kb * 128, dst + i * 1024);
             }
         };
-        auto compute = [&](int slot, int kb) {
-            const uint8_t *src = ring + slot * STAGE_BYTES;
-            const float wsg = s_ws[0][kb], wsu = s_ws[1][kb];
-            v8i ag[NP], au[NP];
+        int slot_w = 0, slot_r = 0;
 #pragma unroll
-            for (int pr = 0; pr < NP; pr++) {
-                ag[pr] = read_tile(src + (2 * pr) * 2048);
-                au[pr] = read_tile(src + (2 * pr + 1) * 2048);
-            }
+        for (int j = 0; j < S - 1; j++) {
+            issue(j / TPK, j % TPK, slot_w);
+            slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
+        }
+        __syncthreads();   // s_xs is complete
+        v8i bfrag[TM];
+        for (int kb = 0; kb < nk; kb++) {
+            const float wsg = s_sc[kb], wsu = s_sc[kItemKBlocks + kb];
+            float sg[TM], su[TM];
 #pragma unroll
             for (int t = 0; t < TM; t++) {
-                const v8i b = cat(bst[slot].b[t][0], bst[slot].b[t][1]);
-                const float sg = wsg * bst[slot].xs[t];
-                const float su = wsu * bst[slot].xs[t];
+                const float xs = s_xs[t * 16 + n][kb];
+                sg[t] = wsg * xs;
+                su[t] = wsu * xs;
+            }
 #pragma unroll
-                for (int pr = 0; pr < NP; pr++) {
-                    accg[pr][t] += mfma_fp8(ag[pr], b) * sg;
-                    accu[pr][t] += mfma_fp8(au[pr], b) * su;
+            for (int a = 0; a < TPK; a++) {
+                issue(kb + (a + S - 1) / TPK, (a + S - 1) % TPK, slot_w);
+                slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
+                __builtin_amdgcn_sched_barrier(0);
+                wait_vmcnt<2 * (S - 1)>();
+                const v8i frag = read_tile(ring + slot_r * 2048);
+                slot_r = slot_r + 1 == S ? 0 : slot_r + 1;
+                if (a < TM) {
+                    bfrag[a < TM ? a : 0] = frag;
+                } else {
+                    const int pr = (a - TM) >> 1;
+#pragma unroll
+                    for (int t = 0; t < TM; t++) {
+                        if (((a - TM) & 1) == 0)
+                            accg[pr < NP ? pr : 0][t] += mfma_fp8(frag, bfrag[t]) * sg[t];
+                        else
+                            accu[pr < NP ? pr : 0][t] += mfma_fp8(frag, bfrag[t]) * su[t];
+                    }
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
-        };
-        pipeline<STAGES, LPS>(nk, issue, compute);
+        }
+        drain_vmem();
+        TRACE_MARK;
 
         if (s.ks > 1) {
-            // K-split: add the valid tokens' partial sums into h[u]; the last arrival takes the totals back
-            float *h_u = s.h + (size_t)u * s.bm_pad * 256;
+            // K-split: store the valid tokens' partial sums to this item's slice; the last arrival adds the slices up
+            const size_t slice = (size_t)s.bm_pad * 256;
+            float *h_u = s.hpart + (size_t)u * s.ks * slice;
+            const int my_off = n * 256 + wave * (RW / 2) + 4 * q;
 #pragma unroll
             for (int t = 0; t < TM; t++) {
                 if (!r.valid[t]) continue;
 #pragma unroll
                 for (int pr = 0; pr < NP; pr++) {
-                    float *dst = h_u + (t * 16 + n) * 256 + wave * (RW / 2) + pr * 16 + 4 * q;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        atomic_add_f32_agent(dst + j, accg[pr][t][j]);
-                        atomic_add_f32_agent(dst + 128 + j, accu[pr][t][j]);
-                    }
+                    float *dst = h_u + ksp * slice + t * 16 * 256 + my_off + pr * 16;
+                    stg128_agent(dst, accg[pr][t]);
+                    stg128_agent(dst + 128, accu[pr][t]);
                 }
             }
             drain_vmem();
@@ -390,106 +426,132 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 s_bcast[1] = __hip_atomic_fetch_add(&s.arrive[u], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __syncthreads();
             if (s_bcast[1] != s.ks - 1) return;
+            if (tid == 0) store_agent(&s.arrive[u], 0);
 #pragma unroll
             for (int t = 0; t < TM; t++)
 #pragma unroll
                 for (int pr = 0; pr < NP; pr++) {
-                    float *src = h_u + (t * 16 + n) * 256 + wave * (RW / 2) + pr * 16 + 4 * q;
-                    v4i g = {0, 0, 0, 0}, up = {0, 0, 0, 0};
+                    v4f g = {0.f, 0.f, 0.f, 0.f}, up = {0.f, 0.f, 0.f, 0.f};
                     if (r.valid[t]) {
-                        g = ldg128_agent(src);
-                        up = ldg128_agent(src + 128);
+                        const float *src = h_u + t * 16 * 256 + my_off + pr * 16;
+                        for (int k = 0; k < s.ks; k++) {   // fixed order: the sum does not depend on arrival order
+                            const v4i gk = ldg128_agent(src + k * slice);
+                            const v4i uk = ldg128_agent(src + k * slice + 128);
+                            drain_vmem();
+                            g += __builtin_bit_cast(v4f, gk);
+                            up += __builtin_bit_cast(v4f, uk);
+                        }
                     }
-                    drain_vmem();
-                    accg[pr][t] = __builtin_bit_cast(v4f, g);
-                    accu[pr][t] = __builtin_bit_cast(v4f, up);
-                    if (r.valid[t]) {
-                        stg128_agent(src, (v4i){0, 0, 0, 0});
-                        stg128_agent(src + 128, (v4i){0, 0, 0, 0});
-                    }
+                    accg[pr][t] = g;
+                    accu[pr][t] = up;
                 }
-            if (tid == 0) store_agent(&s.arrive[u], 0);
         }
         activate_and_publish(u, accg, accu);
     };
 
     auto down_item = [&](int item) {
-        const int u = item / s.n_cs;
-        const int cs = item - u * s.n_cs;
-        const int mb = u / s.n_ib;
-        const int ib = u - mb * s.n_ib;
-        const int e = p.expert_ids[mb];
+        const int mb = item / s.n_cs;
+        const int cs = item - mb * s.n_cs;
+        const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
         if (e >= 0 && e < p.E) {
-            if (tid == 0) spin_until_ge(&s.flag[u], 1, s.ctl);
-            __syncthreads();
-            const Routing<TM> r = load_routing<TM>(p, mb, n);
-
+            const int n_ib = s.n_ib;
             const int t0 = cs * s.tpi;
             const int t1 = (t0 + s.tpi) < s.n_ct ? (t0 + s.tpi) : s.n_ct;
             const int tpw = s.tpi / WN;
             const int wt0 = t0 + wave * tpw;
-            int wnt = (wt0 + tpw < t1 ? wt0 + tpw : t1) - wt0;   // tiles of this wavefront, may be <= 0
-            // w2 scales of the 128-column blocks this item touches
-            const int blk0 = (t0 * 16) >> 7;
-            const int nblk = (((t1 * 16) - 1) >> 7) - blk0 + 1;
-            for (int i = tid; i < nblk; i += THREADS)
-                s_ws[0][i] = p.w2_scale[((size_t)e * (K >> 7) + blk0 + i) * s.n_ib + ib];
-            __syncthreads();
-
-            v8i ba[TM];
-            float tsc[TM];
-            float *accp[TM];
-            const uint8_t *aq_u = s.aq + (size_t)u * s.bm_pad * 128;
+            const int wng = (wt0 + tpw < t1 ? wt0 + tpw : t1) - wt0;   // 16-column groups of this wavefront, may be <= 0
+            const int wnt = wng > 0 ? wng * n_ib : 0;                  // ring tiles: group-major, slice-minor
+            // weights first: they do not depend on the up phase
+            const uint8_t *gd[2];
 #pragma unroll
-            for (int t = 0; t < TM; t++) {
-                const v4i lo = ldg128_agent(aq_u + (t * 16 + n) * 128 + 16 * q);
-                const v4i hi = ldg128_agent(aq_u + (t * 16 + n) * 128 + 64 + 16 * q);
-                const int sa_bits = load_agent(reinterpret_cast<const int *>(&s.sa[(size_t)u * s.bm_pad + t * 16 + n]));
-                drain_vmem();
-                ba[t] = cat(lo, hi);
-                tsc[t] = __builtin_bit_cast(float, sa_bits) * (p.topk_w[r.slot[t]] * p.scaling);
-                accp[t] = p.acc + (size_t)r.tok[t] * K + 4 * q;
-            }
-            if (wnt > 0) {
-                const uint8_t *gd[2];
+            for (int i = 0; i < 2; i++)
+                gd[i] = p.w2 + ((size_t)e * K + (size_t)(wng > 0 ? wt0 : 0) * 16 + 8 * i + ld_row) * I + 16 * ld_chunk[i];
+            const size_t group_step = (size_t)16 * I;
+            int ig = 0, iib = 0;   // (group, slice) of the next tile to issue
+            auto issue = [&](int slot) {
+                uint8_t *dst = ring + slot * 2048;
+                const bool past_end = ig >= wng;
 #pragma unroll
                 for (int i = 0; i < 2; i++)
-                    gd[i] = p.w2 + ((size_t)e * K + (size_t)wt0 * 16 + 8 * i + ld_row) * I + ib * 128 + 16 * ld_chunk[i];
-                const size_t tile_step = (size_t)16 * I;
-                const int n_st = (wnt + DT - 1) / DT;
-                constexpr int LPS = DT * 2;
-                auto issue = [&](int slot, int st) {
-                    uint8_t *dst = ring + slot * STAGE_BYTES;
+                    dma16<2>(past_end ? dummy : gd[i] + ig * group_step + iib * 128, dst + i * 1024);
+                iib++;
+                if (iib == n_ib) {
+                    iib = 0;
+                    ig++;
+                }
+            };
+            int slot_w = 0, slot_r = 0;
 #pragma unroll
-                    for (int j = 0; j < DT; j++) {
-                        int tile = st * DT + j;
-                        tile = tile < wnt ? tile : wnt - 1;
+            for (int j = 0; j < S - 1; j++) {
+                issue(slot_w);
+                slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
+            }
+            // w2 scales of the 128-column blocks this item touches: s_sc[blk * n_ib + ib]
+            const int blk0 = (t0 * 16) >> 7;
+            const int nblk = (((t1 * 16) - 1) >> 7) - blk0 + 1;
+            for (int i = tid; i < nblk * n_ib; i += THREADS)
+                s_sc[i] = p.w2_scale[((size_t)e * (K >> 7) + blk0) * n_ib + i];
+            const Routing<TM> r = load_routing<TM>(p, mb, n);
+
+            if (tid == 0)
+                for (int ib = 0; ib < n_ib; ib++) spin_until_ge(&s.flag[mb * n_ib + ib], epoch, s.ctl);
+            __syncthreads();
+            TRACE_MARK;
+
+            // requantised activations of all slices -> LDS as operand tiles, their scales -> s_xs[row][ib]
+            for (int i = wave; i < n_ib * TM; i += WN) {
+                const int ib = i / TM, t = i - ib * TM;
+                const uint8_t *src = s.aq + ((size_t)(mb * n_ib + ib) * s.bm_pad + t * 16) * 128;
 #pragma unroll
-                        for (int i = 0; i < 2; i++) dma16_nt(gd[i] + tile * tile_step, dst + j * 2048 + i * 1024);
+                for (int k = 0; k < 2; k++)
+                    dma16<16>(src + (8 * k + ld_row) * 128 + 16 * ld_chunk[k], s_aq + i * 2048 + k * 1024);
+            }
+            for (int i = tid; i < n_ib * TM * 16; i += THREADS) {
+                const int ib = i / (TM * 16), row = i - ib * (TM * 16);
+                const int bits = load_agent(reinterpret_cast<const int *>(&s.sa[(size_t)(mb * n_ib + ib) * s.bm_pad + row]));
+                s_xs[row][ib] = __builtin_bit_cast(float, bits);
+            }
+            float tw[TM];
+            float *yp[TM];
+#pragma unroll
+            for (int t = 0; t < TM; t++) {
+                tw[t] = r.valid[t] ? p.topk_w[r.slot[t]] * p.scaling : 0.f;
+                yp[t] = s.y + (size_t)r.slot[t] * K + 4 * q;
+                if (cs == 0 && wave == 0 && q == 0 && r.valid[t]) store_agent(&s.live[r.slot[t]], epoch);
+            }
+            // everything issued so far (the ring's first S-1 tiles, the activation tiles) has landed
+            drain_vmem();
+            __syncthreads();
+
+            v4f d[TM];
+#pragma unroll
+            for (int t = 0; t < TM; t++) d[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+            int cg = 0, cib = 0;   // (group, slice) of the tile being consumed
+            for (int j = 0; j < wnt; j++) {
+                issue(slot_w);
+                slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
+                __builtin_amdgcn_sched_barrier(0);
+                wait_vmcnt<2 * (S - 1)>();
+                const v8i a = read_tile(ring + slot_r * 2048);
+                slot_r = slot_r + 1 == S ? 0 : slot_r + 1;
+                const int c0 = (wt0 + cg) << 4;
+                const float ws = s_sc[((c0 >> 7) - blk0) * n_ib + cib];
+#pragma unroll
+                for (int t = 0; t < TM; t++) {
+                    const v8i b = read_tile(s_aq + (cib * TM + t) * 2048);
+                    d[t] += mfma_fp8(a, b) * (s_xs[t * 16 + n][cib] * ws);
+                }
+                cib++;
+                if (cib == n_ib) {
+                    cib = 0;
+                    cg++;
+#pragma unroll
+                    for (int t = 0; t < TM; t++) {
+                        if (r.valid[t]) stg128_agent(yp[t] + c0, d[t] * tw[t]);
+                        d[t] = (v4f){0.f, 0.f, 0.f, 0.f};
                     }
-                };
-                auto compute = [&](int slot, int st) {
-                    const uint8_t *src = ring + slot * STAGE_BYTES;
-#pragma unroll
-                    for (int j = 0; j < DT; j++) {
-                        const int tile = st * DT + j;
-                        if (tile < wnt) {
-                            const v8i a = read_tile(src + j * 2048);
-                            const int c0 = (wt0 + tile) << 4;
-                            const float ws = s_ws[0][(c0 >> 7) - blk0];
-#pragma unroll
-                            for (int t = 0; t < TM; t++) {
-                                const v4f d = mfma_fp8(a, ba[t]);
-                                const float sc = tsc[t] * ws;
-                                if (r.valid[t]) {
-#pragma unroll
-                                    for (int jj = 0; jj < 4; jj++) atomic_add_f32_agent(accp[t] + c0 + jj, d[jj] * sc);
-                                }
-                            }
-                        }
-                    }
-                };
-                pipeline<STAGES, LPS>(n_st, issue, compute);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         drain_vmem();
@@ -500,45 +562,36 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     auto fin_item = [&](int f) {
         if (tid == 0) spin_until_ge(&s.ctl->down_done, n_down, s.ctl);
         __syncthreads();
-        const int n4 = (int)(((int64_t)p.M * K) >> 2);
-        const int i = f * FIN_CHUNK + tid;
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int idx = i + k * THREADS;
-            if (idx < n4) {
-                const v4i a_bits = ldg128_agent(reinterpret_cast<const v4f *>(p.acc) + idx);
-                uint2 o = reinterpret_cast<uint2 *>(p.out)[idx];
+        TRACE_MARK;
+        const int t = f / s.n_fc;
+        const int c = (f - t * s.n_fc) * kFinCols + tid * 4;
+        if (tid < kFinCols / 4 && c < K) {
+            v4f sum = {0.f, 0.f, 0.f, 0.f};
+            for (int sl = 0; sl < p.top_k; sl++) {   // slot order: the sum does not depend on anything but the inputs
+                const int slot = t * p.top_k + sl;
+                if (load_agent(&s.live[slot]) != epoch) continue;
+                const v4i bits = ldg128_agent(s.y + (size_t)slot * K + c);
                 drain_vmem();
-                const v4f a = __builtin_bit_cast(v4f, a_bits);
-                const float o0 = __builtin_bit_cast(float, o.x << 16), o1 = __builtin_bit_cast(float, o.x & 0xffff0000u);
-                const float o2 = __builtin_bit_cast(float, o.y << 16), o3 = __builtin_bit_cast(float, o.y & 0xffff0000u);
-                o.x = pack_bf16x2(o0 + a[0], o1 + a[1]);
-                o.y = pack_bf16x2(o2 + a[2], o3 + a[3]);
-                reinterpret_cast<uint2 *>(p.out)[idx] = o;
-                reinterpret_cast<v4f *>(p.acc)[idx] = (v4f){0.f, 0.f, 0.f, 0.f};
+                sum += __builtin_bit_cast(v4f, bits);
             }
-        }
-        // this item's share of the per-unit state: nothing reads it any more
-        const int upf = (n_units + s.n_fin - 1) / s.n_fin;
-        const int u0 = f * upf;
-        const int u1 = (u0 + upf) < n_units ? (u0 + upf) : n_units;
-        for (int u = u0 + tid; u < u1; u += THREADS) s.flag[u] = 0;
-        if (u1 > u0) {
-            const int aq16 = s.bm_pad * 8;   // 16-byte pieces of aq per unit
-            v4i *aq = reinterpret_cast<v4i *>(s.aq + (size_t)u0 * s.bm_pad * 128);
-            for (int i = tid; i < (u1 - u0) * aq16; i += THREADS) aq[i] = (v4i){0, 0, 0, 0};
-            float *sa = s.sa + (size_t)u0 * s.bm_pad;
-            for (int i = tid; i < (u1 - u0) * s.bm_pad; i += THREADS) sa[i] = 0.f;
+            uint2 *op = reinterpret_cast<uint2 *>(p.out + (size_t)t * K + c);
+            uint2 o = *op;
+            const float o0 = __builtin_bit_cast(float, o.x << 16), o1 = __builtin_bit_cast(float, o.x & 0xffff0000u);
+            const float o2 = __builtin_bit_cast(float, o.y << 16), o3 = __builtin_bit_cast(float, o.y & 0xffff0000u);
+            o.x = pack_bf16x2(o0 + sum[0], o1 + sum[1]);
+            o.y = pack_bf16x2(o2 + sum[2], o3 + sum[3]);
+            *op = o;
         }
     };
 
     // ---- work queue ---------------------------------------------------------------------------------------
     if (tid == 0) s_bcast[0] = __hip_atomic_fetch_add(&s.ctl->head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
-    int item = s_bcast[0];
+    int item = __builtin_amdgcn_readfirstlane(s_bcast[0]);
     while (item < total) {
         int next = 0;
         if (tid == 0) next = __hip_atomic_fetch_add(&s.ctl->head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        TRACE_BEGIN;
         if (item < n_up)
             up_item(item);
         else if (item < n_up + n_down)
@@ -546,9 +599,10 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         else
             fin_item(item - n_up - n_down);
         __syncthreads();
+        TRACE_END(item < n_up ? 1 : (item < n_up + n_down ? 2 : 3), item);
         if (tid == 0) s_bcast[0] = next;
         __syncthreads();
-        item = s_bcast[0];
+        item = __builtin_amdgcn_readfirstlane(s_bcast[0]);
     }
     if (tid == 0) {
         const int left = __hip_atomic_fetch_add(&s.ctl->done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -556,34 +610,12 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             store_agent(&s.ctl->head, 0);
             store_agent(&s.ctl->done, 0);
             store_agent(&s.ctl->down_done, 0);
+            store_agent(&s.ctl->epoch, epoch);
         }
     }
 }
 
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
-
-struct Layout {
-    size_t ctl, acc, arrive, flag, sa, aq, h, total;
-    int units, bm_pad;
-};
-
-Layout make_layout(int M, int K, int N, int sorted_num, int block_m)
-{
-    Layout L;
-    L.bm_pad = (block_m + 15) / 16 * 16;
-    const size_t n_mb = ((size_t)sorted_num + block_m - 1) / block_m;
-    L.units = (int)(n_mb * (N / 256));
-    size_t off = 0;
-    L.ctl = off; off = align_up(off + sizeof(StreamCtl));
-    L.acc = off; off = align_up(off + (size_t)M * K * sizeof(float));
-    L.arrive = off; off = align_up(off + (size_t)L.units * sizeof(int));
-    L.flag = off; off = align_up(off + (size_t)L.units * sizeof(int));
-    L.sa = off; off = align_up(off + (size_t)L.units * L.bm_pad * sizeof(float));
-    L.aq = off; off = align_up(off + (size_t)L.units * L.bm_pad * 128);
-    L.h = off; off = align_up(off + (size_t)L.units * L.bm_pad * 256 * sizeof(float));
-    L.total = off;
-    return L;
-}
 
 int env_int(const char *name, int dflt)
 {
@@ -591,45 +623,118 @@ int env_int(const char *name, int dflt)
     return e ? atoi(e) : dflt;
 }
 
+// Everything the host decides about one launch; a pure function of the sizes (and of the tuning overrides in the
+// environment), so the workspace query and the launch agree.
+struct HostPlan {
+    bool ok;
+    int bm_pad, n_ib, nkb, n_ct, n_mb_max, units;
+    int kbpi, ks, tpi, n_cs, n_fc;
+    size_t off_sa, off_aq, off_hpart, off_y, total;
+};
+
+HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
+{
+    HostPlan h = {};
+    h.bm_pad = (block_m + 15) / 16 * 16;
+    h.n_ib = N / 256;
+    h.nkb = K / 128;
+    h.n_ct = K / 16;
+    const int64_t rows = (int64_t)M * top_k;
+    // a live row block holds at least one (token, slot) row, so there are at most M*top_k of them
+    int64_t n_mb_max = ((int64_t)sorted_num + block_m - 1) / block_m;
+    if (n_mb_max > rows) n_mb_max = rows;
+    h.n_mb_max = (int)n_mb_max;
+    const int64_t units = n_mb_max * h.n_ib;
+    h.ok = block_m <= 32 && h.n_ib <= kMaxIb && units <= kMaxUnits && rows <= kMaxSlots &&
+           rows * (int64_t)K * 4 <= ((int64_t)1 << 30);
+    if (!h.ok) return h;
+    h.units = (int)units;
+
+    // Item sizes: aim at ~4 items per workgroup slot (2 per CU on a 256-CU part), 64 KiB .. 512 KiB of weights each.
+    const int slots = 512;
+    int64_t mb_est = (rows < E ? rows : E) + rows / block_m;
+    if (mb_est > n_mb_max) mb_est = n_mb_max;
+    const int64_t unit_bytes = (int64_t)256 * K + (int64_t)K * 128;
+    int64_t target = mb_est * h.n_ib * unit_bytes / ((int64_t)slots * 4);
+    if (target < (64 << 10)) target = 64 << 10;
+    if (target > (512 << 10)) target = 512 << 10;
+    int kbpi = (int)((target + (1 << 14)) / (1 << 15));   // 32 KiB of w1 per K block
+    kbpi = env_int("ALPHA_MOE_KBPI", kbpi);
+    if (kbpi < 1) kbpi = 1;
+    if (kbpi > h.nkb) kbpi = h.nkb;
+    if (kbpi > kItemKBlocks) kbpi = kItemKBlocks;
+    h.ks = (h.nkb + kbpi - 1) / kbpi;
+    h.kbpi = (h.nkb + h.ks - 1) / h.ks;                    // even split
+    h.ks = (h.nkb + h.kbpi - 1) / h.kbpi;
+    // a DOWN item reads all n_ib slices of its columns: 2 KiB * n_ib per 16-column tile
+    int tpi = (int)(target / (2048 * h.n_ib)) / 16 * 16;
+    tpi = env_int("ALPHA_MOE_TPI", tpi);
+    if (tpi < 16) tpi = 16;
+    tpi = (tpi + 15) / 16 * 16;
+    if (tpi > (h.n_ct + 15) / 16 * 16) tpi = (h.n_ct + 15) / 16 * 16;
+    if (tpi / 8 * h.n_ib > 1024) tpi = 1024 / h.n_ib * 8 / 16 * 16;   // w2 scales of one item fit s_sc
+    h.n_cs = (h.n_ct + tpi - 1) / tpi;
+    h.tpi = ((h.n_ct + h.n_cs - 1) / h.n_cs + 15) / 16 * 16;   // even split, whole multiples of 16 tiles
+    h.n_cs = (h.n_ct + h.tpi - 1) / h.tpi;
+    h.n_fc = (K + kFinCols - 1) / kFinCols;
+
+    size_t off = align_up(kPrefixBytes);
+    h.off_sa = off; off = align_up(off + (size_t)h.units * h.bm_pad * sizeof(float));
+    h.off_aq = off; off = align_up(off + (size_t)h.units * h.bm_pad * 128);
+    h.off_hpart = off; off = align_up(off + (h.ks > 1 ? (size_t)h.units * h.ks * h.bm_pad * 256 * sizeof(float) : 0));
+    h.off_y = off; off = align_up(off + (size_t)rows * K * sizeof(float));
+    h.total = off;
+    return h;
+}
+
 typedef void (*StreamFn)(const StreamPlan);
 
 struct Variant {
     StreamFn fn;
-    int lds_bytes;
+    int ring_bytes;
     int threads;
+    int tm;
 };
 
-template <int TM, int WN, int ST>
+template <int TM, int WN, int S>
 Variant variant()
 {
-    return Variant{moe_stream_kernel<TM, WN, ST>, 256 * 128 * ST, WN * 64};
+    return Variant{moe_stream_kernel<TM, WN, S>, WN * S * 2048, WN * 64, TM};
 }
 
-template <int TM, int WN>
-Variant pick_stages(int stages)
+// `stages` sizes the LDS ring: 16 KiB per workgroup per stage, i.e. S = 8 * stages / WN tiles of 2 KiB per
+// wavefront (at least 2).  Up to 4 stages, two workgroups share a CU's 160 KiB of LDS.
+template <int TM>
+Variant pick_ring(int wn, int stages)
 {
-    switch (stages) {
-    case 1: return variant<TM, WN, 1>();
-    case 2: return variant<TM, WN, 2>();
-    case 3: return variant<TM, WN, 3>();
-    default: return variant<TM, WN, 4>();   // 4 x 32 KiB of ring is what 160 KiB of LDS holds
+    int tiles = 8 * stages / wn;
+    if (tiles < 2) tiles = 2;
+    if (wn == 4) {
+        switch (tiles) {
+        case 2: return variant<TM, 4, 2>();
+        case 4: return variant<TM, 4, 4>();
+        case 6: return variant<TM, 4, 6>();
+        case 8: return variant<TM, 4, 8>();
+        default: return variant<TM, 4, 10>();
+        }
+    }
+    switch (tiles) {
+    case 2: return variant<TM, 8, 2>();
+    case 3: return variant<TM, 8, 3>();
+    case 4: return variant<TM, 8, 4>();
+    default: return variant<TM, 8, 5>();
     }
 }
 
-Variant pick(int tm, int wn, int stages)
-{
-    if (tm == 1) return wn == 4 ? pick_stages<1, 4>(stages) : pick_stages<1, 8>(stages);
-    return wn == 4 ? pick_stages<2, 4>(stages) : pick_stages<2, 8>(stages);
-}
+Variant pick(int tm, int wn, int stages) { return tm == 1 ? pick_ring<1>(wn, stages) : pick_ring<2>(wn, stages); }
 
 // Workgroups of this variant the current device keeps resident at once; the attribute and occupancy queries run
-// once per (variant, device).
-hipError_t resident_slots(const Variant &v, int *slots)
+// once per (variant, LDS size, device).
+hipError_t resident_slots(const Variant &v, int lds_bytes, int *slots)
 {
     struct Entry {
         StreamFn fn;
-        int dev;
-        int slots;
+        int dev, lds, slots;
     };
     static std::mutex mu;
     static std::vector<Entry> cache;
@@ -638,7 +743,7 @@ hipError_t resident_slots(const Variant &v, int *slots)
     if (err != hipSuccess) return err;
     std::lock_guard<std::mutex> lock(mu);
     for (const Entry &e : cache)
-        if (e.fn == v.fn && e.dev == dev) {
+        if (e.fn == v.fn && e.dev == dev && e.lds == lds_bytes) {
             *slots = e.slots;
             return hipSuccess;
         }
@@ -646,83 +751,84 @@ hipError_t resident_slots(const Variant &v, int *slots)
     err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (err != hipSuccess) return err;
     err = hipFuncSetAttribute(reinterpret_cast<const void *>(v.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              v.lds_bytes);
+                              128 << 10);
     if (err != hipSuccess) return err;
     int occ = 0;
     err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void *>(v.fn), v.threads,
-                                                       v.lds_bytes);
+                                                       lds_bytes);
     if (err != hipSuccess) return err;
     if (occ < 1) occ = 1;
     *slots = cus * occ;
-    cache.push_back(Entry{v.fn, dev, *slots});
+    cache.push_back(Entry{v.fn, dev, lds_bytes, *slots});
     return hipSuccess;
 }
 
 }  // namespace
 
-bool stream_supported(int block_m) { return block_m <= 32; }
-
-size_t stream_workspace_bytes(int M, int K, int N, int sorted_num, int block_m)
+#ifdef ALPHA_MOE_TRACE
+extern "C" int alpha_moe_debug_trace_read(void *dst, int max_records)
 {
-    return make_layout(M, K, N, sorted_num, block_m).total;
+    int n = 0;
+    (void)hipDeviceSynchronize();
+    (void)hipMemcpyFromSymbol(&n, HIP_SYMBOL(g_trace_n), sizeof(int));
+    if (n > max_records) n = max_records;
+    if (n > (1 << 16)) n = 1 << 16;
+    (void)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_trace), (size_t)n * 32);
+    const int zero = 0;
+    (void)hipMemcpyToSymbol(HIP_SYMBOL(g_trace_n), &zero, sizeof(int));
+    return n;
+}
+#endif
+
+size_t stream_prefix_bytes() { return align_up(kPrefixBytes); }
+
+bool stream_supported(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
+{
+    return make_plan(top_k, M, K, N, E, sorted_num, block_m).ok;
+}
+
+size_t stream_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
+{
+    return make_plan(top_k, M, K, N, E, sorted_num, block_m).total;
 }
 
 hipError_t launch_stream(const MoeParams &p, int warp_n, int stages, void *workspace, hipStream_t stream)
 {
-    const Layout L = make_layout(p.M, p.K, p.N, p.sorted_num, p.block_m);
+    const HostPlan h = make_plan(p.top_k, p.M, p.K, p.N, p.E, p.sorted_num, p.block_m);
+    if (!h.ok) return hipErrorInvalidValue;
     uint8_t *ws = static_cast<uint8_t *>(workspace);
     StreamPlan s;
     s.p = p;
-    s.p.acc = reinterpret_cast<float *>(ws + L.acc);
-    s.ctl = reinterpret_cast<StreamCtl *>(ws + L.ctl);
-    s.arrive = reinterpret_cast<int *>(ws + L.arrive);
-    s.flag = reinterpret_cast<int *>(ws + L.flag);
-    s.sa = reinterpret_cast<float *>(ws + L.sa);
-    s.aq = ws + L.aq;
-    s.h = reinterpret_cast<float *>(ws + L.h);
-    s.bm_pad = L.bm_pad;
-    s.n_ib = p.N / 256;
-    s.nkb = p.K / 128;
-    s.n_ct = p.K / 16;
-    s.n_mb_max = (p.sorted_num + p.block_m - 1) / p.block_m;
+    s.ctl = reinterpret_cast<StreamCtl *>(ws);
+    s.arrive = reinterpret_cast<int *>(ws + kOffArrive);
+    s.flag = reinterpret_cast<int *>(ws + kOffFlag);
+    s.live = reinterpret_cast<int *>(ws + kOffLive);
+    s.sa = reinterpret_cast<float *>(ws + h.off_sa);
+    s.aq = ws + h.off_aq;
+    s.hpart = reinterpret_cast<float *>(ws + h.off_hpart);
+    s.y = reinterpret_cast<float *>(ws + h.off_y);
+    s.bm_pad = h.bm_pad;
+    s.n_ib = h.n_ib;
+    s.nkb = h.nkb;
+    s.n_ct = h.n_ct;
+    s.n_mb_max = h.n_mb_max;
+    s.kbpi = h.kbpi;
+    s.ks = h.ks;
+    s.tpi = h.tpi;
+    s.n_cs = h.n_cs;
+    s.n_fc = h.n_fc;
 
     const Variant v = pick((p.block_m + 15) / 16, warp_n, stages);
-
+    const int lds_bytes = v.ring_bytes + h.n_ib * v.tm * 2048;
     int slots = 0;
-    const hipError_t err = resident_slots(v, &slots);
+    const hipError_t err = resident_slots(v, lds_bytes, &slots);
     if (err != hipSuccess) return err;
 
-    // Item sizes: aim at ~4 items per resident workgroup, between 64 KiB and 512 KiB of weights each.
-    const int64_t rows = (int64_t)p.M * p.top_k;
-    int64_t mb_est = (rows < p.E ? rows : p.E) + rows / p.block_m;
-    if (mb_est > s.n_mb_max) mb_est = s.n_mb_max;
-    const int64_t unit_bytes = (int64_t)256 * p.K + (int64_t)p.K * 128;
-    int64_t target = mb_est * s.n_ib * unit_bytes / ((int64_t)slots * 4);
-    if (target < (64 << 10)) target = 64 << 10;
-    if (target > (512 << 10)) target = 512 << 10;
-    int kbpi = (int)((target + (1 << 14)) / (1 << 15));   // 32 KiB of w1 per K block
-    kbpi = env_int("ALPHA_MOE_KBPI", kbpi);
-    if (kbpi < 1) kbpi = 1;
-    if (kbpi > s.nkb) kbpi = s.nkb;
-    s.ks = (s.nkb + kbpi - 1) / kbpi;
-    s.kbpi = (s.nkb + s.ks - 1) / s.ks;                    // even split
-    s.ks = (s.nkb + s.kbpi - 1) / s.kbpi;
-    int tpi = (int)(target / (16 * 2048)) * 16;            // 2 KiB of w2 per tile, whole multiples of 16 tiles
-    tpi = env_int("ALPHA_MOE_TPI", tpi);
-    if (tpi < 16) tpi = 16;
-    tpi = (tpi + 15) / 16 * 16;
-    if (tpi > (s.n_ct + 15) / 16 * 16) tpi = (s.n_ct + 15) / 16 * 16;
-    s.n_cs = (s.n_ct + tpi - 1) / tpi;
-    s.tpi = ((s.n_ct + s.n_cs - 1) / s.n_cs + 15) / 16 * 16;   // even split, whole multiples of 16 tiles
-    s.n_cs = (s.n_ct + s.tpi - 1) / s.tpi;
-    const int64_t n4 = (int64_t)p.M * p.K / 4;
-    s.n_fin = (int)((n4 + v.threads * 4 - 1) / (v.threads * 4));
-
-    const int64_t max_items = (int64_t)L.units * (s.ks + s.n_cs) + s.n_fin;
+    const int64_t max_items = (int64_t)h.units * h.ks + (int64_t)h.n_mb_max * h.n_cs + (int64_t)p.M * h.n_fc;
     int grid = env_int("ALPHA_MOE_GRID", slots);
     if (grid > max_items) grid = (int)max_items;
     if (grid < 1) grid = 1;
-    hipLaunchKernelGGL(v.fn, dim3((unsigned)grid), dim3((unsigned)v.threads), v.lds_bytes, stream, s);
+    hipLaunchKernelGGL(v.fn, dim3((unsigned)grid), dim3((unsigned)v.threads), lds_bytes, stream, s);
     return hipGetLastError();
 }
 

@@ -20,9 +20,9 @@
 
 namespace {
 
-// Scratch for the C ABI, one buffer per (device, stream): zero-filled when created, left zero-filled by every
-// call, so the steady state allocates and clears nothing (the first call on a stream does both: warm the
-// operator up once before capturing it into a HIP graph).
+// Scratch for the C ABI, one buffer per (device, stream): zero-filled when created and maintained by the library
+// afterwards, so the steady state allocates and clears nothing (the first call on a stream, or the first with a
+// larger problem, does both: warm the operator up once before capturing it into a HIP graph).
 at::Tensor workspace_for(const at::Device &dev, hipStream_t stream, size_t bytes)
 {
     static std::mutex mu;
@@ -92,8 +92,9 @@ void fused_moe_w8a8_up_down(const at::Tensor &x, const at::Tensor &x_scale, cons
     const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(dev);
     hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
 
-    const size_t ws_bytes = alpha_moe_workspace_bytes(static_cast<int>(M), static_cast<int>(K), static_cast<int>(N),
-                                                      static_cast<int>(sorted_num), static_cast<int>(block_m));
+    const size_t ws_bytes =
+        alpha_moe_workspace_bytes(static_cast<int>(top_k), static_cast<int>(M), static_cast<int>(K), static_cast<int>(N),
+                                  static_cast<int>(E), static_cast<int>(sorted_num), static_cast<int>(block_m));
     at::Tensor ws = workspace_for(dev, stream, ws_bytes);
 
     const int rc = alpha_moe_fused_moe_w8a8_up_down(

@@ -50,10 +50,11 @@ enum alpha_moe_status {
  *   block_m          8..128 step 8     must equal the block size sorted_token_ids was built with
  *   (block_n, warp_n) (64,4) or (32,8) wavefronts per workgroup = warp_n, w1 rows per wavefront = block_n
  *   stages           1..5              K-blocks of loads kept in flight per wavefront
- *   workspace        device scratch of at least alpha_moe_workspace_bytes(M, K, N, sorted_num, block_m) bytes,
- *                    256-byte aligned.  It must be ZERO-FILLED before its first use; every call leaves it zero-filled
- *                    again, so one buffer can be kept for the life of the process and serve calls of any sizes it is
- *                    large enough for.  Calls that share a workspace must be ordered on one stream.
+ *   workspace        device scratch of at least alpha_moe_workspace_bytes(top_k, M, K, N, num_experts, sorted_num,
+ *                    block_m) bytes, 256-byte aligned.  It must be ZERO-FILLED once, before its first use; after
+ *                    that its contents belong to the library (self-resetting counters, per-launch epochs) and the
+ *                    same buffer serves any number of calls, of any sizes it is large enough for, without being
+ *                    cleared.  Calls that share a workspace must be ordered on one stream.
  */
 int alpha_moe_fused_moe_w8a8_up_down(
     const uint8_t *x, const float *x_scale,
@@ -67,7 +68,7 @@ int alpha_moe_fused_moe_w8a8_up_down(
     float scaling_factor, void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
 
 /* Bytes of scratch the call above needs for these sizes (0 if any is not positive). */
-size_t alpha_moe_workspace_bytes(int M, int K, int N, int sorted_num, int block_m);
+size_t alpha_moe_workspace_bytes(int top_k, int M, int K, int N, int num_experts, int sorted_num, int block_m);
 
 /*
  * The argument checks of the call above without touching the device: returns the status the launch would

@@ -23,7 +23,7 @@ def run_op(P, block_m, block_n, warp_n, stages, out=None, scaling=None, via="tor
                                                    stages, scaling)
     else:
         stream = torch.cuda.current_stream().cuda_stream
-        ws_bytes = alpha_moe.c_abi.alpha_moe_workspace_bytes(P.M, P.shape.K, P.shape.N, s_ids.numel(), block_m)
+        ws_bytes = alpha_moe.c_abi.alpha_moe_workspace_bytes(P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E, s_ids.numel(), block_m)
         ws = workspace if workspace is not None else torch.zeros(ws_bytes, dtype=torch.uint8, device=P.x.device)
         assert ws.numel() >= ws_bytes
         rc = alpha_moe.c_abi.alpha_moe_fused_moe_w8a8_up_down(
@@ -32,8 +32,7 @@ def run_op(P, block_m, block_n, warp_n, stages, out=None, scaling=None, via="tor
             P.topk_weights.data_ptr(), P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E, s_ids.numel(), block_m,
             block_n, warp_n, stages, float(scaling), ws.data_ptr(), ws.numel(), stream)
         assert rc == 0, alpha_moe.c_abi.alpha_moe_status_string(rc)
-        torch.cuda.synchronize()
-        assert int(ws.count_nonzero()) == 0, "the call must leave its workspace zero-filled"
+
 
     torch.cuda.synchronize()
     return out

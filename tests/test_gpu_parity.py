@@ -32,7 +32,7 @@ def test_c_abi_workspace_is_reusable_without_clearing(c1):
     """One zero-filled workspace, many calls with different knobs (and so different kernels and layouts inside it)."""
     import alpha_moe
     P, ref = c1
-    sizes = [alpha_moe.c_abi.alpha_moe_workspace_bytes(P.M, P.shape.K, P.shape.N, P.align(bm)[0].numel(), bm)
+    sizes = [alpha_moe.c_abi.alpha_moe_workspace_bytes(P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E, P.align(bm)[0].numel(), bm)
              for bm in (8, 16, 32, 64)]
     ws = torch.zeros(max(sizes), dtype=torch.uint8, device=DEV)
     for bm, bn, wn, st in [(16, 64, 4, 2), (16, 64, 4, 2), (8, 32, 8, 3), (64, 64, 4, 2), (32, 32, 8, 1), (16, 64, 4, 4)]:
