@@ -81,6 +81,7 @@ struct StreamPlan {
     int kbpi, ks;    // K blocks per UP item, UP items per unit
     int tpi, n_cs;   // 16-column tiles per DOWN item, DOWN items per row block
     int n_fc;        // FIN items per token
+    int lag;         // row blocks between a block's UP items and its DOWN items in the queue
     int bm_pad;
 };
 
@@ -250,6 +251,15 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         return cat(*reinterpret_cast<const v4i *>(tile + frag_lo), *reinterpret_cast<const v4i *>(tile + frag_hi));
     };
 
+    // The next item is taken from the queue when the current one has finished streaming (its atomic's round trip
+    // hides behind the item's epilogue).  Taking it any earlier lets busy workgroups sit on items that idle ones
+    // could already run.
+    int next_item = -1;
+    auto fetch_next = [&]() {
+        if (tid == 0 && next_item < 0)
+            next_item = __hip_atomic_fetch_add(&s.ctl->head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    };
+
     // SwiGLU + per-token amax over the 128 columns + FP8 requant of one unit, from accumulators in the MFMA layout.
     auto activate_and_publish = [&](int u, v4f (&accg)[NP][TM], v4f (&accu)[NP][TM]) {
 #pragma unroll
@@ -402,6 +412,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        fetch_next();
         drain_vmem();
         TRACE_MARK;
 
@@ -547,13 +558,20 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                     cg++;
 #pragma unroll
                     for (int t = 0; t < TM; t++) {
+#if defined(EXP_NO_STORE)
+                        if (r.valid[t] && c0 < 0) stg128_agent(yp[t] + c0, d[t] * tw[t]);
+#elif defined(EXP_PLAIN_STORE)
+                        if (r.valid[t]) *reinterpret_cast<v4f *>(yp[t] + c0) = d[t] * tw[t];
+#else
                         if (r.valid[t]) stg128_agent(yp[t] + c0, d[t] * tw[t]);
+#endif
                         d[t] = (v4f){0.f, 0.f, 0.f, 0.f};
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
+        fetch_next();
         drain_vmem();
         __syncthreads();
         if (tid == 0) __hip_atomic_fetch_add(&s.ctl->down_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -567,12 +585,19 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         const int c = (f - t * s.n_fc) * kFinCols + tid * 4;
         if (tid < kFinCols / 4 && c < K) {
             v4f sum = {0.f, 0.f, 0.f, 0.f};
-            for (int sl = 0; sl < p.top_k; sl++) {   // slot order: the sum does not depend on anything but the inputs
-                const int slot = t * p.top_k + sl;
-                if (load_agent(&s.live[slot]) != epoch) continue;
-                const v4i bits = ldg128_agent(s.y + (size_t)slot * K + c);
+            // slot order: the sum depends on nothing but the inputs.  Eight rows are in flight at a time.
+            for (int s0 = 0; s0 < p.top_k; s0 += 8) {
+                v4i bits[8];
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    const int slot = t * p.top_k + s0 + k;
+                    const bool on = s0 + k < p.top_k && load_agent(&s.live[slot]) == epoch;
+                    bits[k] = (v4i){0, 0, 0, 0};
+                    if (on) bits[k] = ldg128_agent(s.y + (size_t)slot * K + c);
+                }
                 drain_vmem();
-                sum += __builtin_bit_cast(v4f, bits);
+#pragma unroll
+                for (int k = 0; k < 8; k++) sum += __builtin_bit_cast(v4f, bits[k]);
             }
             uint2 *op = reinterpret_cast<uint2 *>(p.out + (size_t)t * K + c);
             uint2 o = *op;
@@ -585,22 +610,51 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     };
 
     // ---- work queue ---------------------------------------------------------------------------------------
+    // Order: round r holds the UP items of row block r followed by the DOWN items of row block r - lag, so the two
+    // kinds overlap, a DOWN item is taken long after the UP items it waits for, and only `lag` blocks' worth of
+    // DOWN items remain when the UP items run out.  FIN items come last.
+    const int per_up = s.n_ib * s.ks, per_down = s.n_cs;
+    const int lag = s.lag < n_mb ? s.lag : n_mb;
+    const int head_items = lag * per_up;                          // rounds 0 .. lag-1: UP only
+    const int mid_items = (n_mb - lag) * (per_up + per_down);     // rounds lag .. n_mb-1: UP then DOWN
+    auto run_item = [&](int item) -> int {
+        if (item >= n_up + n_down) {
+            fin_item(item - n_up - n_down);
+            return 3;
+        }
+        int up = -1, down = -1;
+        if (item < head_items) {
+            up = item;
+        } else if (item < head_items + mid_items) {
+            const int i = item - head_items;
+            const int round = i / (per_up + per_down);
+            const int off = i - round * (per_up + per_down);
+            if (off < per_up)
+                up = (lag + round) * per_up + off;
+            else
+                down = round * per_down + (off - per_up);
+        } else {
+            down = (n_mb - lag) * per_down + (item - head_items - mid_items);
+        }
+        if (up >= 0) {
+            up_item(up);
+            return 1;
+        }
+        down_item(down);
+        return 2;
+    };
     if (tid == 0) s_bcast[0] = __hip_atomic_fetch_add(&s.ctl->head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     int item = __builtin_amdgcn_readfirstlane(s_bcast[0]);
     while (item < total) {
-        int next = 0;
-        if (tid == 0) next = __hip_atomic_fetch_add(&s.ctl->head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         TRACE_BEGIN;
-        if (item < n_up)
-            up_item(item);
-        else if (item < n_up + n_down)
-            down_item(item - n_up);
-        else
-            fin_item(item - n_up - n_down);
+        next_item = -1;
+        const int kind = run_item(item);
+        (void)kind;
+        fetch_next();   // paths that did not get there themselves (skipped blocks, FIN items)
         __syncthreads();
-        TRACE_END(item < n_up ? 1 : (item < n_up + n_down ? 2 : 3), item);
-        if (tid == 0) s_bcast[0] = next;
+        TRACE_END(kind, item);
+        if (tid == 0) s_bcast[0] = next_item;
         __syncthreads();
         item = __builtin_amdgcn_readfirstlane(s_bcast[0]);
     }
@@ -628,7 +682,7 @@ int env_int(const char *name, int dflt)
 struct HostPlan {
     bool ok;
     int bm_pad, n_ib, nkb, n_ct, n_mb_max, units;
-    int kbpi, ks, tpi, n_cs, n_fc;
+    int kbpi, ks, tpi, n_cs, n_fc, lag;
     size_t off_sa, off_aq, off_hpart, off_y, total;
 };
 
@@ -650,14 +704,16 @@ HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int bl
     if (!h.ok) return h;
     h.units = (int)units;
 
-    // Item sizes: aim at ~4 items per workgroup slot (2 per CU on a 256-CU part), 64 KiB .. 512 KiB of weights each.
+    // Item sizes (from sweeps on MI355X, DeepSeek-V3 shard, M = 1..64): about one UP item per workgroup slot and
+    // K split, between 128 KiB and 1 MiB of w1 each - smaller items drown in their fixed cost (a dozen dependent
+    // memory round trips), larger ones leave a long tail; DOWN items of at most 256 KiB of w2.
     const int slots = 512;
     int64_t mb_est = (rows < E ? rows : E) + rows / block_m;
     if (mb_est > n_mb_max) mb_est = n_mb_max;
     const int64_t unit_bytes = (int64_t)256 * K + (int64_t)K * 128;
-    int64_t target = mb_est * h.n_ib * unit_bytes / ((int64_t)slots * 4);
-    if (target < (64 << 10)) target = 64 << 10;
-    if (target > (512 << 10)) target = 512 << 10;
+    int64_t target = mb_est * h.n_ib * unit_bytes / slots;
+    if (target < (128 << 10)) target = 128 << 10;
+    if (target > (1 << 20)) target = 1 << 20;
     int kbpi = (int)((target + (1 << 14)) / (1 << 15));   // 32 KiB of w1 per K block
     kbpi = env_int("ALPHA_MOE_KBPI", kbpi);
     if (kbpi < 1) kbpi = 1;
@@ -667,7 +723,8 @@ HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int bl
     h.kbpi = (h.nkb + h.ks - 1) / h.ks;                    // even split
     h.ks = (h.nkb + h.kbpi - 1) / h.kbpi;
     // a DOWN item reads all n_ib slices of its columns: 2 KiB * n_ib per 16-column tile
-    int tpi = (int)(target / (2048 * h.n_ib)) / 16 * 16;
+    const int64_t down_target = target < (256 << 10) ? target : (256 << 10);
+    int tpi = (int)(down_target / (2048 * h.n_ib)) / 16 * 16;
     tpi = env_int("ALPHA_MOE_TPI", tpi);
     if (tpi < 16) tpi = 16;
     tpi = (tpi + 15) / 16 * 16;
@@ -677,6 +734,11 @@ HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int bl
     h.tpi = ((h.n_ct + h.n_cs - 1) / h.n_cs + 15) / 16 * 16;   // even split, whole multiples of 16 tiles
     h.n_cs = (h.n_ct + h.tpi - 1) / h.tpi;
     h.n_fc = (K + kFinCols - 1) / kFinCols;
+    // how many row blocks later a block's DOWN items enter the queue than its UP items
+    // (measured: overlapping the two kinds lowers the total rate - DOWN items stream less efficiently than UP items -
+    // so by default the lag is "all blocks", i.e. UP items first, then DOWN items)
+    h.lag = env_int("ALPHA_MOE_LAG", 1 << 30);
+    if (h.lag < 1) h.lag = 1;
 
     size_t off = align_up(kPrefixBytes);
     h.off_sa = off; off = align_up(off + (size_t)h.units * h.bm_pad * sizeof(float));
@@ -817,6 +879,7 @@ hipError_t launch_stream(const MoeParams &p, int warp_n, int stages, void *works
     s.tpi = h.tpi;
     s.n_cs = h.n_cs;
     s.n_fc = h.n_fc;
+    s.lag = h.lag;
 
     const Variant v = pick((p.block_m + 15) / 16, warp_n, stages);
     const int lds_bytes = v.ring_bytes + h.n_ib * v.tm * 2048;
