@@ -1,0 +1,192 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused W8A8 MoE operator on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--M 64] [--shape ds]
+
+A "step" is one call of torch.ops.alpha_moe.fused_moe_w8a8_up_down on a DeepSeek-V3-like single-GPU TP shard
+(E=257 incl. the fused shared expert, top_k=9, K=7168, I=256, FP8 e4m3 with 128x128 block scales) with all inputs
+resident in HBM.  The headline is M=64 decode; M = 1, 4, 16 are measured in the same run and reported under "per_M".
+Consecutive steps rotate through several copies of the weights and several routings so that a step never finds its
+weights in the 256 MiB Infinity Cache; `out` is not re-zeroed inside the timed region (the operator adds into it).
+
+Prints ONE JSON line: the driver's contract fields plus
+  "roofline":     algorithmic HBM bytes per launch / average launch duration (HIP events on the launch stream)
+  "cpu_baseline": the CPU oracle (oracle/moe_oracle.py, a port of the reference maths) timed on the host cores
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "alpha-moe_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
+FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
+DEFAULT_KNOBS = {"block_m": 16, "block_n": 32, "warp_n": 8, "stages": 5}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--shape", default="ds", choices=["ds", "qn", "q3", "c1"])
+    ap.add_argument("--M", type=int, default=64, help="tokens of the headline measurement")
+    ap.add_argument("--also-M", type=int, nargs="*", default=None, help="other token counts reported under per_M")
+    ap.add_argument("--replicas", type=int, default=6, help="copies of the weights rotated through")
+    ap.add_argument("--config", default=None, help="tuning table (JSON of jit_moe.py); default: shipped table or built-in knobs")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    return ap.parse_args()
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this operator is a single-GPU kernel on one tensor-parallel shard and has no "
+              f"multi-GPU path (asked for --gpus {args.gpus}).", file=sys.stderr)
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    import alpha_moe  # noqa: F401  fails loudly if the HIP libraries are not built
+    from alpha_moe_python.utils import get_best_config
+    from alpha_moe_python.workloads import SHAPES, Weights, make_problem, make_weights
+
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    shape = SHAPES[args.shape]
+    cfg_path = args.config or os.path.join(ROOT, "alpha-moe_amd", "configs", f"moe_jit_{shape.E}_{shape.N}_{shape.K}.json")
+
+    def knobs_for(M):
+        if os.path.exists(cfg_path):
+            return dict(get_best_config(cfg_path, M)), os.path.relpath(cfg_path, ROOT)
+        return dict(DEFAULT_KNOBS), "built-in"
+
+    W0 = make_weights(shape, device=dev, seed=0)
+    replicas = [W0]
+    for _ in range(max(1, args.replicas) - 1):
+        replicas.append(Weights(shape, W0.w1.clone(), W0.w1_scale.clone(), W0.w2.clone(), W0.w2_scale.clone()))
+    n_routings = 8
+
+    def prepare(M):
+        """Problems (routing + activations) for M tokens, one per routing seed, each bound to one weight replica."""
+        knobs, src = knobs_for(M)
+        calls, byts, flops = [], [], []
+        for i in range(n_routings):
+            W = replicas[i % len(replicas)]
+            P = make_problem(W, M, seed=i)
+            s_ids, e_ids, total = P.align(knobs["block_m"])
+            out = torch.zeros((M, shape.K), dtype=torch.bfloat16, device=dev)
+            byts.append(P.algorithmic_bytes())
+            flops.append(P.algorithmic_flops())
+
+            def call(P=P, W=W, s_ids=s_ids, e_ids=e_ids, total=total, out=out):
+                torch.ops.alpha_moe.fused_moe_w8a8_up_down(
+                    P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids, total, P.topk_weights, out,
+                    shape.top_k, knobs["block_m"], knobs["block_n"], knobs["warp_n"], knobs["stages"],
+                    shape.scaling_factor)
+            calls.append(call)
+        return calls, statistics.mean(byts), statistics.mean(flops), knobs, src
+
+    def measure(M, steps, warmup):
+        calls, B, F, knobs, src = prepare(M)
+        for i in range(warmup):
+            calls[i % len(calls)]()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            calls[i % len(calls)]()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+        # per-launch device time: HIP events on the launch stream (torch's current stream) around every call
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for i in range(steps):
+            evs[i][0].record()
+            calls[i % len(calls)]()
+            evs[i][1].record()
+        torch.cuda.synchronize()
+        dev_ms = [a.elapsed_time(b) for a, b in evs]
+        return {"M": M, "ms_per_step": wall_ms, "launch_us_mean": statistics.mean(dev_ms) * 1e3,
+                "launch_us_median": statistics.median(dev_ms) * 1e3, "launch_us_min": min(dev_ms) * 1e3,
+                "bytes": B, "flops": F, "knobs": knobs, "knobs_from": src}
+
+    head = measure(args.M, args.steps, args.warmup)
+    others = args.also_M if args.also_M is not None else [m for m in (1, 4, 16, 64) if m != args.M]
+    per_M = {}
+    for m in [args.M] + list(others):
+        r = head if m == args.M else measure(m, max(20, args.steps // 2), args.warmup)
+        t_us = r["launch_us_mean"]
+        per_M[str(m)] = {
+            "us_per_layer": round(r["ms_per_step"] * 1e3, 2), "launch_us_mean": round(t_us, 2),
+            "launch_us_median": round(r["launch_us_median"], 2),
+            "algorithmic_MB": round(r["bytes"] / 1e6, 1), "GB_per_s": round(r["bytes"] / t_us / 1e3, 1),
+            "hbm_frac": round(r["bytes"] / t_us / 1e3 / HBM_PEAK_GBS, 4),
+            "TFLOP_per_s": round(r["flops"] / t_us / 1e6, 2),
+            "mfma_frac": round(r["flops"] / t_us / 1e6 / FP8_PEAK_TFLOPS, 5), "knobs": r["knobs"]}
+
+    achieved = head["bytes"] / head["launch_us_mean"] / 1e3   # GB/s
+    result = {
+        "metric": "us_per_fused_moe_layer",
+        "value": round(head["ms_per_step"] * 1e3, 2),
+        "unit": "us",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(head["ms_per_step"], 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3",
+        "data": "synthetic",
+        "config": {"workload": f"{shape.name}_decode_M{args.M}: E={shape.E} top_k={shape.top_k} K={shape.K} I={shape.I} "
+                               f"fp8 e4m3 128x128 block scales, {len(replicas)} weight copies x {n_routings} routings rotated",
+                   "M": args.M, "knobs": head["knobs"], "knobs_from": head["knobs_from"]},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "moe_stream_kernel", "algorithmic_bytes_per_launch": int(head["bytes"]),
+                     "launch_us_mean": round(head["launch_us_mean"], 2)},
+        "per_M": per_M,
+    }
+
+    if not args.no_cpu_baseline:
+        # the CPU port of the reference maths on the same bits, on this box's host cores (checker, not product)
+        from oracle import moe_oracle as O
+        torch.set_num_threads(os.cpu_count() or 1)
+        Wc = Weights(shape, W0.w1.cpu(), W0.w1_scale.cpu(), W0.w2.cpu(), W0.w2_scale.cpu())
+        P = make_problem(W0, args.M, seed=0)
+        knobs = head["knobs"]
+        s_ids, e_ids, total = P.align(knobs["block_m"])
+        out = torch.zeros((args.M, shape.K), dtype=torch.bfloat16, device=dev)
+        torch.ops.alpha_moe.fused_moe_w8a8_up_down(P.x, P.x_scale, W0.w1, W0.w1_scale, W0.w2, W0.w2_scale, s_ids, e_ids, total,
+                                                   P.topk_weights, out, shape.top_k, knobs["block_m"], knobs["block_n"],
+                                                   knobs["warp_n"], knobs["stages"], shape.scaling_factor)
+        torch.cuda.synchronize()
+        cpu_args = [t.cpu() for t in (P.x, P.x_scale)] + [Wc.w1, Wc.w1_scale, Wc.w2, Wc.w2_scale] + \
+                   [t.cpu() for t in (s_ids, e_ids, total, P.topk_weights)]
+        zero = torch.zeros((args.M, shape.K), dtype=torch.bfloat16)
+        times = []
+        ref = None
+        t_budget = time.perf_counter()
+        for _ in range(3):
+            t0 = time.perf_counter()
+            ref = O.fused_moe_oracle(*cpu_args, zero, shape.top_k, knobs["block_m"], shape.scaling_factor)
+            times.append(time.perf_counter() - t0)
+            if time.perf_counter() - t_budget > 30:
+                break
+        result["cpu_baseline"] = {"value": round(statistics.median(times) * 1e6, 1), "unit": "us", "cores": torch.get_num_threads(),
+                                  "kind": "port", "sample": f"same call as the headline (M={args.M}, routing seed 0), "
+                                                            f"median of {len(times)} runs of oracle/moe_oracle.py (torch fp32)"}
+        result["parity"] = O.error_metrics(out, ref)
+
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
