@@ -24,6 +24,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "alpha-moe_amd"))
 sys.path.insert(0, ROOT)
 
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy of known size), for the
+# configurations that were profiled: profiles/moe_stream_kernel_ds_decode_M64_hbm_traffic.md
+MEASURED_TRAFFIC_BYTES = {("ds", 64): 1302.5e6}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
 DEFAULT_KNOBS = {"block_m": 16, "block_n": 32, "warp_n": 8, "stages": 5}
@@ -40,6 +43,9 @@ def parse_args():
     ap.add_argument("--replicas", type=int, default=6, help="copies of the weights rotated through")
     ap.add_argument("--config", default=None, help="tuning table (JSON of jit_moe.py); default: shipped table or built-in knobs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy three times: a kernel of known traffic to scale "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings by")
     return ap.parse_args()
 
 
@@ -116,6 +122,14 @@ def main():
                 "launch_us_median": statistics.median(dev_ms) * 1e3, "launch_us_min": min(dev_ms) * 1e3,
                 "bytes": B, "flops": F, "knobs": knobs, "knobs_from": src}
 
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.int32, device=dev)   # 1 GiB read + 1 GiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     head = measure(args.M, args.steps, args.warmup)
     others = args.also_M if args.also_M is not None else [m for m in (1, 4, 16, 64) if m != args.M]
     per_M = {}
@@ -148,7 +162,8 @@ def main():
                                f"fp8 e4m3 128x128 block scales, {len(replicas)} weight copies x {n_routings} routings rotated",
                    "M": args.M, "knobs": head["knobs"], "knobs_from": head["knobs_from"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.shape, args.M)),
                      "kernel": "moe_stream_kernel", "algorithmic_bytes_per_launch": int(head["bytes"]),
                      "launch_us_mean": round(head["launch_us_mean"], 2)},
         "per_M": per_M,
