@@ -24,13 +24,26 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.path.join(ROCM, "bin", "hipcc")
 
 # packed-fp32 VALU forms are switched off for every kernel in this library
-HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+# Per-source extras.  The tile kernel scales every matrix-instruction result into vector-register accumulators, so
+# the results must land in vector registers, not in accumulation registers that only a copy can read.
+HIP_SOURCES = {
+    "moe_api.hip": [],
+    "moe_direct.hip": [],
+    "moe_stream.hip": [],
+    "moe_tile.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
 
 
 def run(cmd):
     print("+", " ".join(cmd), flush=True)
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    finish(cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True))
+
+
+def finish(cmd, proc):
+    out, _ = proc.communicate()
+    res = subprocess.CompletedProcess(cmd, proc.returncode, out)
     lines = [l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l]
     if lines:
         print("\n".join(lines), flush=True)
@@ -39,8 +52,18 @@ def run(cmd):
 
 
 def build_hip():
-    srcs = [os.path.join(CSRC, f) for f in ("moe_api.hip", "moe_direct.hip", "moe_stream.hip")]
-    run([HIPCC, *HIP_FLAGS, "-o", HIP_LIB, *srcs])
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    jobs, objs = [], []
+    for src, extra in HIP_SOURCES.items():   # one compiler process per source, all at once
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        cmd = [HIPCC, *HIP_FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+        print("+", " ".join(cmd), flush=True)
+        jobs.append((cmd, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs.append(obj)
+    for cmd, proc in jobs:
+        finish(cmd, proc)
+    run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", HIP_LIB, *objs])
     return HIP_LIB
 
 

@@ -8,7 +8,7 @@ using namespace alpha_moe;
 
 namespace {
 
-// ALPHA_MOE_PATH=direct|stream forces one kernel family (for experiments); default: streaming kernel where it applies.
+// ALPHA_MOE_PATH=direct|stream|tile forces one kernel family where it applies (for experiments).
 int forced_path()
 {
     static const int v = [] {
@@ -16,15 +16,27 @@ int forced_path()
         if (!e) return 0;
         if (!strcmp(e, "direct")) return 1;
         if (!strcmp(e, "stream")) return 2;
+        if (!strcmp(e, "tile")) return 3;
         return 0;
     }();
     return v;
 }
 
-bool use_stream(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
+enum Path { kDirect, kStream, kTile };
+
+// Streaming kernel for row blocks of at most 32 rows (decode), tile kernel above (prefill); the direct kernel is the
+// fallback for shapes neither takes.
+Path choose_path(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
 {
-    if (!stream_supported(top_k, M, K, N, E, sorted_num, block_m)) return false;
-    return forced_path() != 1;
+    const bool s_ok = stream_supported(top_k, M, K, N, E, sorted_num, block_m);
+    const bool t_ok = tile_supported(top_k, M, K, N, E, sorted_num, block_m);
+    const int f = forced_path();
+    if (f == 1) return kDirect;
+    if (f == 2 && s_ok) return kStream;
+    if (f == 3 && t_ok) return kTile;
+    if (s_ok) return kStream;
+    if (t_ok) return kTile;
+    return kDirect;
 }
 
 }  // namespace
@@ -53,7 +65,11 @@ extern "C" size_t alpha_moe_workspace_bytes(int top_k, int M, int K, int N, int 
     const size_t stream = stream_supported(top_k, M, K, N, num_experts, sorted_num, block_m)
                               ? stream_workspace_bytes(top_k, M, K, N, num_experts, sorted_num, block_m)
                               : 0;
-    return direct > stream ? direct : stream;
+    const size_t tile = tile_supported(top_k, M, K, N, num_experts, sorted_num, block_m)
+                            ? tile_workspace_bytes(top_k, M, K, N, num_experts, sorted_num, block_m)
+                            : 0;
+    const size_t m = direct > stream ? direct : stream;
+    return m > tile ? m : tile;
 }
 
 extern "C" int alpha_moe_fused_moe_w8a8_up_down(const uint8_t *x, const float *x_scale, const uint8_t *w,
@@ -85,8 +101,11 @@ extern "C" int alpha_moe_fused_moe_w8a8_up_down(const uint8_t *x, const float *x
 
     hipStream_t hs = static_cast<hipStream_t>(stream);
     hipError_t err;
-    if (use_stream(top_k, M, K, N, num_experts, sorted_num, block_m)) {
+    const Path path = choose_path(top_k, M, K, N, num_experts, sorted_num, block_m);
+    if (path == kStream) {
         err = launch_stream(p, warp_n, stages, workspace, hs);
+    } else if (path == kTile) {
+        err = launch_tile(p, workspace, hs);
     } else {
         err = launch_zero_acc(p, hs);
         if (err == hipSuccess) err = launch_direct(p, warp_n, stages, hs);

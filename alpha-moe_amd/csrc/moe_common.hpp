@@ -93,6 +93,29 @@ __device__ __forceinline__ void atomic_add_f32(float *addr, float v)
     __builtin_amdgcn_global_atomic_fadd_f32(reinterpret_cast<gptr>(reinterpret_cast<uintptr_t>(addr)), v);
 }
 
+// ---- workspace prefix shared by the kernel families --------------------------------------------------------
+// The first kPrefixBytes of the workspace are zero-initialised by the caller once and maintained by the kernels:
+// counters return to zero by themselves, flags are stamped with a launch epoch that only ever grows.  Its size
+// does not depend on the problem, so calls of different sizes can share one buffer.
+constexpr int kMaxUnits = 1 << 16;   // most (row block, slice) units of one streaming launch
+constexpr int kMaxSlots = 1 << 18;   // most (token, slot) rows whose results go through per-slot rows
+
+struct StreamCtl {
+    int head;        // streaming kernel: next work item
+    int done;        // streaming kernel: workgroups that have left
+    int epoch;       // completed launches on this workspace (any kernel family)
+    int down_done;   // streaming kernel: finished DOWN items of this launch
+    int error;       // sticky: a bounded wait ran out
+    int fin_done;    // tile kernels: reduce-kernel workgroups that have left
+    int pad[58];
+};
+static_assert(sizeof(StreamCtl) == 256, "control block is one 256-byte line group");
+
+constexpr size_t kOffArrive = 256;
+constexpr size_t kOffFlag = kOffArrive + sizeof(int) * kMaxUnits;
+constexpr size_t kOffLive = kOffFlag + sizeof(int) * kMaxUnits;
+constexpr size_t kPrefixBytes = kOffLive + sizeof(int) * kMaxSlots;
+
 // ---- host-side launchers, one per kernel family (each in its own translation unit) -------------------------
 
 // One workgroup per (block of block_m sorted rows, 128-column intermediate slice), weights HBM -> VGPR.
@@ -109,5 +132,12 @@ size_t stream_prefix_bytes();
 bool stream_supported(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
 size_t stream_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
 hipError_t launch_stream(const MoeParams &p, int warp_n, int stages, void *workspace, hipStream_t stream);
+
+
+// Tiled kernel for large batches: one workgroup per row block, token tiles shared through LDS, all I/128 slices in
+// one workgroup, per-slot bf16 result rows reduced by a second kernel.
+bool tile_supported(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
+size_t tile_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
+hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream);
 
 }  // namespace alpha_moe

@@ -47,25 +47,7 @@ namespace {
 
 constexpr int kItemKBlocks = 64;     // most K blocks one UP item covers
 constexpr int kMaxIb = 16;           // most 128-column slices of the intermediate (I <= 2048)
-constexpr int kMaxUnits = 1 << 16;   // most (row block, slice) units of one launch
-constexpr int kMaxSlots = 1 << 18;   // most (token, slot) rows of one launch
 constexpr int kFinCols = 1024;       // output columns per FIN item
-
-struct StreamCtl {
-    int head;        // next work item
-    int done;        // workgroups that have left
-    int epoch;       // completed launches on this workspace
-    int down_done;   // finished DOWN items of this launch
-    int error;       // sticky: a bounded wait ran out
-    int pad[59];
-};
-static_assert(sizeof(StreamCtl) == 256, "control block is one 256-byte line group");
-
-// zero-initialised, self-maintaining part of the workspace; its size does not depend on the problem
-constexpr size_t kOffArrive = 256;
-constexpr size_t kOffFlag = kOffArrive + sizeof(int) * kMaxUnits;
-constexpr size_t kOffLive = kOffFlag + sizeof(int) * kMaxUnits;
-constexpr size_t kPrefixBytes = kOffLive + sizeof(int) * kMaxSlots;
 
 struct StreamPlan {
     MoeParams p;
@@ -558,13 +540,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                     cg++;
 #pragma unroll
                     for (int t = 0; t < TM; t++) {
-#if defined(EXP_NO_STORE)
-                        if (r.valid[t] && c0 < 0) stg128_agent(yp[t] + c0, d[t] * tw[t]);
-#elif defined(EXP_PLAIN_STORE)
-                        if (r.valid[t]) *reinterpret_cast<v4f *>(yp[t] + c0) = d[t] * tw[t];
-#else
                         if (r.valid[t]) stg128_agent(yp[t] + c0, d[t] * tw[t]);
-#endif
                         d[t] = (v4f){0.f, 0.f, 0.f, 0.f};
                     }
                 }

@@ -1,0 +1,518 @@
+// Fused W8A8 MoE, "tile" kernel for large batches: one workgroup (4 wavefronts) per row block of block_m sorted rows.
+//
+// Up/gate projection.  The workgroup walks the I/128 slices of the intermediate one after the other.  For a slice it
+// contracts its 256 interleaved w1 rows against the block's tokens over all of K, one 128-byte K block per step.
+// Every operand reaches the matrix cores through LDS, filled by direct-to-LDS loads that cover whole 128-byte lines:
+// measured on MI355X, a compute unit takes ~38 GB/s from L2 when a load instruction touches 16 rows x 64 bytes (the
+// matrix-operand register layout) and ~100 GB/s when it touches 8 rows x 128 bytes, and at full matrix rate a
+// 128-token block needs ~110 GB/s.  Each wavefront owns 64 weight rows (4 operand tiles) and streams them through a
+// private 3-stage ring; the token tiles (16 tokens x 128 bytes, gathered through the routing) and their scales go
+// through a 3-stage ring shared by the four wavefronts, with one workgroup barrier per step.  A wavefront issues
+// 4 x TM matrix instructions per step; the 4 multiply-adds that scale a 16x16 product into the fp32 accumulators are
+// placed right behind the NEXT matrix instruction so that vector and matrix pipes overlap (75% of the FP8 peak for
+// this loop in isolation against 35% when the compiler orders it).
+//
+// SwiGLU and the FP8 requantisation of the 128-column group happen in registers (cross-wavefront amax through LDS).
+// LDS is full of rings at that point, so the block_m x 128 FP8 tile is parked in a scratch area of the workspace (it
+// stays in L2) in operand-tile layout and fetched back into LDS, where the rings were, once all slices are done.
+//
+// Down projection.  64 output columns at a time (4 operand tiles of w2 rows, again a private ring per wavefront; no
+// barriers), all slices, all token tiles.  The w2 rows of a tile are picked so that a lane ends up with 16 adjacent
+// output columns of its token: each valid (token, slot) row is written ONCE, in bf16, as whole 128-byte lines, to
+// y[slot]: top_k result rows per token instead of the top_k * I/128 partial rows the reference's decomposition
+// (fused_moe_w8a8_up_down_acc.cu:676-679,1085-1091) adds into the output.  A second kernel sums a token's live rows
+// in fp32 and rounds into `out` once.  No atomics: at M = 8192 fp32 atomics alone cost 13 ms on MI355X.
+//
+// Workgroups are renumbered so that consecutive row blocks (the blocks of one expert) run on the same XCD and share
+// its L2: the hardware deals workgroup i to XCD i % 8.
+#include "moe_common.hpp"
+
+namespace alpha_moe {
+namespace {
+
+constexpr int kTileMaxIb = 8;        // most 128-column slices of the intermediate (I <= 1024)
+constexpr int kTileMaxKb = 128;      // most 128-byte K blocks (K <= 16384)
+constexpr int kTileMaxW2s = 512;     // most w2 block scales of one expert, (K/128) * (I/128)
+constexpr int kStages = 3;
+constexpr int kARingBytes = 4 * kStages * 8192;   // 4 wavefronts x 3 stages x 4 tiles of 2 KiB
+constexpr int kMaxTailBytes = 48 << 10;           // token-tile ring / requantised tiles next to the weight rings
+
+struct TileParams {
+    MoeParams p;
+    StreamCtl *ctl;
+    int *live;        // [slots] == epoch once y[slot] is written this launch
+    uint16_t *y;      // [slots][K] bf16
+    uint8_t *aqs;     // [row blocks][n_ib][TM] requantised operand tiles of 2 KiB
+    int n_ib, nkb, n_mb_max;
+};
+
+typedef const void __attribute__((address_space(1))) * gptr_t;
+typedef void __attribute__((address_space(3))) * lptr_t;
+
+// memory -> LDS without passing VGPRs: lane l's 16 (4) bytes land at lds + 16 l (4 l); the global address is per lane
+__device__ __forceinline__ void dma16(const void *g, void *lds)
+{
+    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uintptr_t)lds, 16, 0, 0);
+}
+__device__ __forceinline__ void dma4(const void *g, void *lds)
+{
+    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uintptr_t)lds, 4, 0, 0);
+}
+
+// The compiler does not count direct-to-LDS loads; the loops below do.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
+{
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// Workgroup barrier that waits for this wavefront's LDS operations only (__syncthreads would also drain every
+// outstanding global load, and with them the prefetches in flight).
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// One step of a wavefront: 4 weight tiles x TM token tiles, all from LDS.  acc[k][t] += (A_k x B_t) * row[t] * sc[k & 1]
+// with row[] a per-token factor in LDS (16 floats per tile, already offset to this lane's token).  The product of
+// (k, t) is scaled into its accumulator behind the matrix instruction of (k, t + 1).
+template <int TM>
+__device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *b_tiles, const float *row, float sc0,
+                                         float sc1, v4f (&acc)[4][TM], int frag_lo, int frag_hi)
+{
+    auto read_tile = [&](const uint8_t *tile) -> v8i {
+        return cat(*reinterpret_cast<const v4i *>(tile + frag_lo), *reinterpret_cast<const v4i *>(tile + frag_hi));
+    };
+    v8i a[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) a[k] = read_tile(a_tiles + k * 2048);
+    v8i b = read_tile(b_tiles);
+    float f = row[0];
+    v4f prev[4];
+    float p0 = 0.f, p1 = 0.f;
+#pragma unroll
+    for (int t = 0; t < TM; t++) {
+        v8i b_next = b;
+        float f_next = f;
+        if (t + 1 < TM) {
+            b_next = read_tile(b_tiles + (t + 1) * 2048);
+            f_next = row[(t + 1) * 16];
+        }
+        v4f cur[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            cur[k] = mfma_fp8(a[k], b);
+            if (t > 0) acc[k][t - 1] += prev[k] * ((k & 1) ? p1 : p0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) prev[k] = cur[k];
+        p0 = f * sc0;
+        p1 = f * sc1;
+        b = b_next;
+        f = f_next;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) acc[k][TM - 1] += prev[k] * ((k & 1) ? p1 : p0);
+}
+
+// TM: 16-token tiles per row block.
+template <int TM>
+__global__ __launch_bounds__(256) void moe_tile_kernel(const TileParams s)
+{
+    constexpr int THREADS = 256;
+    constexpr int XT = (TM + 3) / 4;          // token tiles each wavefront gathers per K block
+    constexpr int XOPS = 3 * XT;              // its vector-memory operations for that: 2 tile halves + 16 scales
+    constexpr int AOPS = 8;                   // 4 weight tiles x 2 halves
+    constexpr int OPS1 = AOPS + XOPS;
+
+    // [4 wavefronts][3 stages][4 tiles] weight rings | [3 stages][TM] token tiles; the requantised tiles [n_ib][TM]
+    // later take the place of the token tiles
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds_dyn[];
+    __shared__ __attribute__((aligned(1024))) uint8_t s_dummy[2048 + 64];
+    __shared__ float s_xs[kStages][TM * 16];
+    __shared__ float s_ws[2][kTileMaxKb];
+    __shared__ float s_amax[4][TM * 16];
+    __shared__ float s_sa[kTileMaxIb][TM * 16];
+    __shared__ float s_w2s[kTileMaxW2s];
+    __shared__ int s_tok[TM * 16];
+
+    const MoeParams &p = s.p;
+    // consecutive row blocks on one XCD: workgroup i runs on XCD i % 8
+    int n_live = (p.ntpp[0] + p.block_m - 1) / p.block_m;
+    n_live = n_live < s.n_mb_max ? n_live : s.n_mb_max;
+    const int per_xcd = (n_live + 7) >> 3;
+    const int mb = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per_xcd || mb >= n_live) return;
+    const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
+    if (e < 0 || e >= p.E) return;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15;
+    const int q = lane >> 4;
+    const int K = p.K, I = p.N >> 1;
+    const int n_ib = s.n_ib, nkb = s.nkb;
+    const int epoch = __builtin_amdgcn_readfirstlane(s.ctl->epoch) + 1;
+    uint8_t *a_ring = lds_dyn + wave * (kStages * 8192);
+    uint8_t *xbuf = lds_dyn + kARingBytes;
+
+    // operand fragment of lane (n, q): chunks q and q+4 of row n; chunk c of row r sits at position c ^ ((r >> 1) & 7)
+    const int f_n = (n >> 1) & 7;
+    const int frag_lo = n * 128 + 16 * (q ^ f_n);
+    const int frag_hi = n * 128 + 16 * ((q ^ f_n) ^ 4);
+    // direct-to-LDS load h of a tile: lane l fills position l & 7 of row 8h + l / 8
+    const int ld_row = lane >> 3;
+    int ld_chunk[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) ld_chunk[h] = 16 * ((lane & 7) ^ (((8 * h + ld_row) >> 1) & 7));
+
+    // ---- routing ---------------------------------------------------------------------------------------------
+    int slot[TM];
+    bool valid[TM];
+#pragma unroll
+    for (int t = 0; t < TM; t++) {
+        const int row = t * 16 + n;
+        const int idx = mb * p.block_m + row;
+        int id = -1;
+        if (row < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
+        valid[t] = id >= 0 && id / p.top_k < p.M;
+        slot[t] = valid[t] ? id : 0;
+        if (wave == 0 && q == 0 && valid[t]) s.live[slot[t]] = epoch;
+    }
+    if (tid < TM * 16) {
+        const int idx = mb * p.block_m + tid;
+        int id = -1;
+        if (tid < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
+        const int tk = id / p.top_k;
+        s_tok[tid] = (id >= 0 && tk < p.M) ? tk : 0;
+    }
+    for (int i = tid; i < (K >> 7) * n_ib; i += THREADS) s_w2s[i] = p.w2_scale[(size_t)e * (K >> 7) * n_ib + i];
+    __syncthreads();
+
+    // token-tile gather: wavefront w loads tiles w and w+4 (a dummy where the block has no such tile)
+    const uint8_t *gx[XT][2];
+    const float *gxs[XT];
+    int xdst[XT];       // byte offset of the tile inside a ring stage, or -1: dummy
+#pragma unroll
+    for (int k = 0; k < XT; k++) {
+        const int t = wave + 4 * k;
+        const bool real = t < TM;
+        xdst[k] = real ? t * 2048 : -1;
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+            gx[k][h] = p.x + (size_t)s_tok[real ? t * 16 + 8 * h + ld_row : 0] * K + ld_chunk[h];
+        gxs[k] = p.x_scale + (size_t)s_tok[real ? t * 16 + (lane & 15) : 0] * nkb;
+    }
+    auto issue_x = [&](int kb, int stage) {   // XOPS operations
+        const int kc = kb < nkb ? kb : nkb - 1;
+#pragma unroll
+        for (int k = 0; k < XT; k++) {
+            uint8_t *dst = xdst[k] >= 0 ? xbuf + stage * (TM * 2048) + xdst[k] : s_dummy;
+            dma16(gx[k][0] + (size_t)kc * 128, dst);
+            dma16(gx[k][1] + (size_t)kc * 128, dst + 1024);
+            float *sdst = xdst[k] >= 0 ? &s_xs[stage][(wave + 4 * k) * 16] : reinterpret_cast<float *>(s_dummy + 2048);
+            if (lane < 16) dma4(gxs[k] + kc, sdst);
+        }
+    };
+
+    v4f acc[4][TM];
+    for (int ib = 0; ib < n_ib; ib++) {
+        // this slice's gate (row 2*ib) and up (row 2*ib+1) scale rows
+        {
+            const float *ws_rows = p.w_scale + ((size_t)e * (p.N >> 7) + 2 * ib) * nkb;
+            for (int i = tid; i < 2 * nkb; i += THREADS) s_ws[i >= nkb][i >= nkb ? i - nkb : i] = ws_rows[i];
+        }
+        // Weight rows of this wavefront: tile a = (pair a / 2, gate | up a % 2); matrix row r of the tile is slab row
+        // pair * 32 + (r / 8) * 16 + r % 8 (+ 8 for up), so load h of a tile covers slab rows ... + 16 h + lane / 8.
+        const uint8_t *wbase = p.w + ((size_t)e * p.N + ib * 256 + wave * 64 + ld_row) * K;
+        auto issue_a = [&](int kb, int stage) {   // AOPS operations
+            const int kc = kb < nkb ? kb : nkb - 1;
+            uint8_t *dst = a_ring + stage * 8192;
+#pragma unroll
+            for (int a = 0; a < 4; a++)
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                    dma16(wbase + (size_t)((a >> 1) * 32 + h * 16 + 8 * (a & 1)) * K + (size_t)kc * 128 + ld_chunk[h],
+                          dst + a * 2048 + h * 1024);
+        };
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int t = 0; t < TM; t++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+        // Per wavefront the loads of step kb are issued two steps ahead.  Step kb: wait for the own loads of kb (those of
+        // kb + 1 stay in flight), meet the others (their token tiles of kb have landed, and everybody is done reading
+        // stage (kb + 2) % 3), refill that stage, compute.
+        __syncthreads();   // s_ws written; everybody is done with the previous slice
+        issue_a(0, 0);
+        issue_x(0, 0);
+        issue_a(1, 1);
+        issue_x(1, 1);
+        for (int kb0 = 0; kb0 < nkb; kb0 += kStages) {
+#pragma unroll
+            for (int h = 0; h < kStages; h++) {
+                const int kb = kb0 + h;
+                if (kb < nkb) {
+                    wait_vmcnt<OPS1>();
+                    lds_barrier();
+                    issue_a(kb + 2, (h + 2) % kStages);
+                    issue_x(kb + 2, (h + 2) % kStages);
+                    __builtin_amdgcn_sched_barrier(0);
+                    mma_step<TM>(a_ring + h * 8192, xbuf + h * (TM * 2048), &s_xs[h][n], s_ws[0][kb], s_ws[1][kb], acc,
+                                 frag_lo, frag_hi);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+        wait_vmcnt<0>();
+
+        // ---- SwiGLU, per-token amax over the slice's 128 columns, FP8 requant into operand tiles (scratch) ---------
+#pragma unroll
+        for (int t = 0; t < TM; t++) {
+            float m = 0.f;
+#pragma unroll
+            for (int pr = 0; pr < 2; pr++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const float a = swiglu_bf16(acc[2 * pr][t][j], acc[2 * pr + 1][t][j]);
+                    acc[2 * pr][t][j] = a;
+                    m = fmaxf(m, fabsf(a));
+                }
+            m = fmaxf(m, __shfl_xor(m, 16));
+            m = fmaxf(m, __shfl_xor(m, 32));
+            if (q == 0) s_amax[wave][t * 16 + n] = m;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < TM; t++) {
+            float m = kAmaxFloor;
+#pragma unroll
+            for (int wv = 0; wv < 4; wv++) m = fmaxf(m, s_amax[wv][t * 16 + n]);
+            const float s_a = m / kFp8Max;
+            uint8_t *tile = s.aqs + ((size_t)(mb * n_ib + ib) * TM + t) * 2048;
+#pragma unroll
+            for (int pr = 0; pr < 2; pr++) {
+                const uint32_t packed =
+                    pack_fp8x4(clamp_fp8(acc[2 * pr][t][0] / s_a), clamp_fp8(acc[2 * pr][t][1] / s_a),
+                               clamp_fp8(acc[2 * pr][t][2] / s_a), clamp_fp8(acc[2 * pr][t][3] / s_a));
+                // columns wave*32 + pr*16 + 4q .. +3 of token n: chunk wave*2 + pr of the row, bytes 4q .. 4q+3 in it
+                *reinterpret_cast<uint32_t *>(tile + n * 128 + 16 * ((wave * 2 + pr) ^ f_n) + 4 * q) = packed;
+            }
+            if (wave == 0 && q == 0) s_sa[ib][t * 16 + n] = s_a;
+        }
+    }
+    // the requantised tiles come back from scratch (L2) into LDS where the token ring was
+    __syncthreads();   // also waits for this wavefront's scratch stores
+    uint8_t *aq = xbuf;
+    for (int i = wave; i < n_ib * TM; i += 4) {
+        const uint8_t *src = s.aqs + ((size_t)mb * n_ib * TM + i) * 2048 + lane * 16;
+        dma16(src, aq + i * 2048);
+        dma16(src + 1024, aq + i * 2048 + 1024);
+    }
+    wait_vmcnt<0>();
+    __syncthreads();
+
+    // ---- down projection: 64 output columns per step group, all slices ---------------------------------------------
+    // Matrix row r of tile k is output column c0 + 16 (r / 4) + 4 k + r % 4, so lane (n, q) collects columns
+    // c0 + 16 q .. c0 + 16 q + 15 of token n over the four tiles.  Load h of a tile: rows 8h + lane / 8.
+    float tw[TM];
+#pragma unroll
+    for (int t = 0; t < TM; t++) tw[t] = valid[t] ? p.topk_w[slot[t]] * p.scaling : 0.f;
+    const int n_groups = K >> 6;
+    const int my_groups = (n_groups - wave + 3) >> 2;   // column groups wave, wave + 4, ...
+    const int n_steps = my_groups * n_ib;               // (group, slice) steps, slice-minor
+    const uint8_t *w2base = p.w2 + ((size_t)e * K + 16 * (lane >> 5) + (ld_row & 3)) * I;
+    int lg = 0, lib = 0;   // (group index, slice) of the next step to load
+    auto issue2 = [&](int stage) {   // AOPS operations
+        const int gc = lg < my_groups ? lg : my_groups - 1;
+        const int c0 = (wave + 4 * gc) << 6;
+        uint8_t *dst = a_ring + stage * 8192;
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                dma16(w2base + (size_t)(c0 + 32 * h + 4 * k) * I + lib * 128 + ld_chunk[h], dst + k * 2048 + h * 1024);
+        lib++;
+        if (lib == n_ib) {
+            lib = 0;
+            lg++;
+        }
+    };
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int t = 0; t < TM; t++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+    int cg = 0, cib = 0;
+    if (n_steps > 0) {
+        issue2(0);
+        issue2(1);
+        for (int s0 = 0; s0 < n_steps; s0 += kStages) {
+#pragma unroll
+            for (int h = 0; h < kStages; h++) {
+                if (s0 + h < n_steps) {
+                    // one younger step of AOPS loads stays in flight; result stores only make this stricter
+                    wait_vmcnt<AOPS>();
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // done reading the stage that is refilled
+                    issue2((h + 2) % kStages);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const int c0 = (wave + 4 * cg) << 6;
+                    const float ws2 = s_w2s[(c0 >> 7) * n_ib + cib];
+                    mma_step<TM>(a_ring + h * 8192, aq + cib * (TM * 2048), &s_sa[cib][n], ws2, ws2, acc, frag_lo, frag_hi);
+                    __builtin_amdgcn_sched_barrier(0);
+                    cib++;
+                    if (cib == n_ib) {
+#pragma unroll
+                        for (int t = 0; t < TM; t++) {
+                            if (valid[t]) {
+                                uint16_t *yp = s.y + (size_t)slot[t] * K + c0 + 16 * q;
+#pragma unroll
+                                for (int half = 0; half < 2; half++) {
+                                    const v4f lo = acc[2 * half][t] * tw[t], hi = acc[2 * half + 1][t] * tw[t];
+                                    v4i o;
+                                    o.x = (int)pack_bf16x2(lo[0], lo[1]);
+                                    o.y = (int)pack_bf16x2(lo[2], lo[3]);
+                                    o.z = (int)pack_bf16x2(hi[0], hi[1]);
+                                    o.w = (int)pack_bf16x2(hi[2], hi[3]);
+                                    *reinterpret_cast<v4i *>(yp + 8 * half) = o;
+                                }
+                            }
+#pragma unroll
+                            for (int a = 0; a < 4; a++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+                        }
+                        cib = 0;
+                        cg++;
+                    }
+                }
+            }
+        }
+        wait_vmcnt<0>();
+    }
+}
+
+// out[t] = bf16(out[t] + sum over the token's live slots of y[slot]); the last workgroup to leave closes the epoch.
+// A unit is (token, 2048 columns): a thread owns 8 columns and keeps up to 8 row loads in flight.  Workgroups stride
+// over the units so that the closing counter sees a few thousand arrivals, not one per unit.
+__global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams s, int chunks_per_token, int n_units)
+{
+    const MoeParams &p = s.p;
+    const int epoch = s.ctl->epoch + 1;
+    for (int unit = blockIdx.x; unit < n_units; unit += gridDim.x) {
+        const int t = unit / chunks_per_token;
+        const int c = (unit - t * chunks_per_token) * 2048 + threadIdx.x * 8;
+        if (c >= p.K) continue;
+        float sum[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        auto add = [&](const v4i v) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                sum[2 * i] += __builtin_bit_cast(float, (uint32_t)v[i] << 16);
+                sum[2 * i + 1] += __builtin_bit_cast(float, (uint32_t)v[i] & 0xffff0000u);
+            }
+        };
+        v4i *op = reinterpret_cast<v4i *>(p.out + (size_t)t * p.K + c);
+        const v4i prior = *op;
+        const int *live = s.live + t * p.top_k;
+        const uint16_t *yrow = s.y + (size_t)t * p.top_k * p.K + c;
+        for (int s0 = 0; s0 < p.top_k; s0 += 8) {   // slot order: the sum depends on nothing but the inputs
+            bool on[8];
+            v4i v[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) on[j] = s0 + j < p.top_k && live[s0 + j] == epoch;
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (on[j]) v[j] = __builtin_nontemporal_load(reinterpret_cast<const v4i *>(yrow + (size_t)(s0 + j) * p.K));
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+                if (on[j]) add(v[j]);
+        }
+        add(prior);
+        v4i o;
+#pragma unroll
+        for (int i = 0; i < 4; i++) o[i] = (int)pack_bf16x2(sum[2 * i], sum[2 * i + 1]);
+        *op = o;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const int left = __hip_atomic_fetch_add(&s.ctl->fin_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (left == (int)gridDim.x - 1) {
+            __hip_atomic_store(&s.ctl->fin_done, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(&s.ctl->epoch, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+int tail_tiles(int n_ib) { return n_ib > kStages ? n_ib : kStages; }
+
+typedef void (*TileFn)(const TileParams);
+
+TileFn pick(int tm)
+{
+    switch (tm) {
+    case 1: return moe_tile_kernel<1>;
+    case 2: return moe_tile_kernel<2>;
+    case 3: return moe_tile_kernel<3>;
+    case 4: return moe_tile_kernel<4>;
+    case 5: return moe_tile_kernel<5>;
+    case 6: return moe_tile_kernel<6>;
+    case 7: return moe_tile_kernel<7>;
+    default: return moe_tile_kernel<8>;
+    }
+}
+
+}  // namespace
+
+bool tile_supported(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
+{
+    (void)E;
+    (void)sorted_num;
+    const int tm = (block_m + 15) / 16;
+    const int n_ib = N / 256;
+    return n_ib <= kTileMaxIb && tail_tiles(n_ib) * tm * 2048 <= kMaxTailBytes && K <= 128 * kTileMaxKb &&
+           (K / 128) * n_ib <= kTileMaxW2s && (int64_t)M * top_k <= kMaxSlots;
+}
+
+size_t tile_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
+{
+    (void)E;
+    const int tm = (block_m + 15) / 16;
+    const size_t n_mb = ((size_t)sorted_num + block_m - 1) / block_m;
+    return align_up(kPrefixBytes) + align_up((size_t)M * top_k * K * sizeof(uint16_t)) +
+           align_up(n_mb * (N / 256) * tm * 2048);
+}
+
+hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
+{
+    uint8_t *ws = static_cast<uint8_t *>(workspace);
+    TileParams s;
+    s.p = p;
+    s.ctl = reinterpret_cast<StreamCtl *>(ws);
+    s.live = reinterpret_cast<int *>(ws + kOffLive);
+    s.y = reinterpret_cast<uint16_t *>(ws + align_up(kPrefixBytes));
+    s.aqs = ws + align_up(kPrefixBytes) + align_up((size_t)p.M * p.top_k * p.K * sizeof(uint16_t));
+    s.n_ib = p.N / 256;
+    s.nkb = p.K / 128;
+    s.n_mb_max = (p.sorted_num + p.block_m - 1) / p.block_m;
+    const int tm = (p.block_m + 15) / 16;
+    const TileFn fn = pick(tm);
+    const int lds_bytes = kARingBytes + tail_tiles(s.n_ib) * tm * 2048;
+    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         kARingBytes + kMaxTailBytes);
+    if (err != hipSuccess) return err;
+    const int grid = (s.n_mb_max + 7) / 8 * 8;
+    hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(256), lds_bytes, stream, s);
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    const int chunks = (p.K + 2047) / 2048;
+    const int n_units = p.M * chunks;
+    hipLaunchKernelGGL(moe_tile_reduce_kernel, dim3((unsigned)(n_units < 4096 ? n_units : 4096)), dim3(256), 0, stream, s,
+                       chunks, n_units);
+    return hipGetLastError();
+}
+
+}  // namespace alpha_moe

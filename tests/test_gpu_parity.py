@@ -118,3 +118,34 @@ def test_deepseek_shard_decode_full_size(ds_weights, M, knobs):
     print(f"case ds M={M} knobs {knobs}", flush=True)
     m = assert_parity(run_op(P, *knobs), oracle_out(P), f"ds M={M} knobs {knobs}")
     print("metrics", m, flush=True)
+
+
+@pytest.mark.parametrize("knobs", [(48, 64, 4, 3), (64, 32, 8, 2), (128, 64, 4, 3)])
+def test_deepseek_shard_prefill_tile_kernel(ds_weights, knobs):
+    """Row blocks above 32 rows go to the tile kernel: M=256 of the DeepSeek-V3 shard against the oracle."""
+    P = make_problem(ds_weights, 256, seed=1)
+    print(f"case ds M=256 knobs {knobs}", flush=True)
+    m = assert_parity(run_op(P, *knobs, via="c_abi"), oracle_out(P), f"ds M=256 knobs {knobs}")
+    print("metrics", m, flush=True)
+
+
+def test_deepseek_shard_prefill_full_size_properties(ds_weights):
+    """M=8192 (73 728 routed rows) is beyond what the oracle finishes in seconds, but a token's result depends on
+    nothing but its own row, routing and the weights: the oracle recomputes a random sample of tokens as a
+    48-token problem and must agree with the corresponding rows.  Two launches agree bit for bit (no atomics), and
+    so do two row-block sizes (the per-slot sums do not depend on which rows share a block)."""
+    from alpha_moe_python.workloads import Problem
+    M = 8192
+    P = make_problem(ds_weights, M, seed=2)
+    print("case ds M=8192 knobs (128, 64, 4, 3)", flush=True)
+    out = run_op(P, 128, 64, 4, 3, via="c_abi")
+    gen = torch.Generator().manual_seed(7)
+    idx = torch.randperm(M, generator=gen)[:48].sort().values.to(DEV)
+    sub = Problem(ds_weights, 48, P.x[idx].contiguous(), P.x_scale[idx].contiguous(), P.topk_ids[idx].contiguous(),
+                  P.topk_weights[idx].contiguous())
+    m = assert_parity(out[idx], oracle_out(sub), "ds M=8192 sampled tokens")
+    print("metrics", m, flush=True)
+    print("case ds M=8192 second launch", flush=True)
+    assert torch.equal(out, run_op(P, 128, 64, 4, 3, via="c_abi"))
+    print("case ds M=8192 knobs (64, 64, 4, 3)", flush=True)
+    assert torch.equal(out, run_op(P, 64, 64, 4, 3, via="c_abi"))
