@@ -1,25 +1,33 @@
-// Fused W8A8 MoE, "tile" kernel for large batches: one workgroup (4 wavefronts) per row block of block_m sorted rows.
+// Fused W8A8 MoE, "tile" kernel for large batches: one workgroup of 8 wavefronts (two per SIMD) per row block of
+// block_m sorted rows.
 //
 // Up/gate projection.  The workgroup walks the I/128 slices of the intermediate one after the other.  For a slice it
 // contracts its 256 interleaved w1 rows against the block's tokens over all of K, one 128-byte K block per step.
 // Every operand reaches the matrix cores through LDS, filled by direct-to-LDS loads that cover whole 128-byte lines:
 // measured on MI355X, a compute unit takes ~38 GB/s from L2 when a load instruction touches 16 rows x 64 bytes (the
 // matrix-operand register layout) and ~100 GB/s when it touches 8 rows x 128 bytes, and at full matrix rate a
-// 128-token block needs ~110 GB/s.  Each wavefront owns 64 weight rows (4 operand tiles) and streams them through a
-// private 3-stage ring; the token tiles (16 tokens x 128 bytes, gathered through the routing) and their scales go
-// through a 3-stage ring shared by the four wavefronts, with one workgroup barrier per step.  A wavefront issues
-// 4 x TM matrix instructions per step; the 4 multiply-adds that scale a 16x16 product into the fp32 accumulators are
-// placed right behind the NEXT matrix instruction so that vector and matrix pipes overlap (75% of the FP8 peak for
-// this loop in isolation against 35% when the compiler orders it).
+// 128-token block needs ~110 GB/s.  Wavefront (w, g) multiplies weight rows 64 w .. 64 w + 63 (4 operand tiles) with
+// token half g; the two wavefronts of a pair w share a 3-stage ring of weight tiles and each loads half of it; the
+// token tiles (16 tokens x 128 bytes, gathered through the routing) and their scales go through a 3-stage ring shared
+// by everybody, one tile per wavefront, with one workgroup barrier per step.  A wavefront issues 4 x TH matrix
+// instructions per step; the 4 multiply-adds that scale a 16x16 product into the fp32 accumulators are placed right
+// behind the NEXT matrix instruction so that vector and matrix pipes overlap (75% of the FP8 peak for this loop in
+// isolation against 35% when the compiler orders it), and the step's loads are spread between them: a direct-to-LDS
+// load blocks the issuing wavefront for 30-60 ns, during which the SIMD's other wavefront computes.
+//
+// What bounds it (measured, M = 8192 on the DeepSeek-V3 shard): a step takes ~1.5 us against 0.43 us of matrix time.
+// A compute unit keeps about 32 KiB of L2 misses in flight whatever the ring depth (two or three stages, one or four
+// wavefronts issuing: same rate), so its load rate is 32 KiB / latency: ~100 GB/s on L2 hits, ~40 GB/s on misses; the
+// first block of an expert misses on all 48 KiB of a step, and the blocks sharing its weights follow at its pace.
 //
 // SwiGLU and the FP8 requantisation of the 128-column group happen in registers (cross-wavefront amax through LDS).
 // LDS is full of rings at that point, so the block_m x 128 FP8 tile is parked in a scratch area of the workspace (it
-// stays in L2) in operand-tile layout and fetched back into LDS, where the rings were, once all slices are done.
+// stays in L2) in operand-tile layout and fetched back into LDS, where the token ring was, once all slices are done.
 //
-// Down projection.  64 output columns at a time (4 operand tiles of w2 rows, again a private ring per wavefront; no
-// barriers), all slices, all token tiles.  The w2 rows of a tile are picked so that a lane ends up with 16 adjacent
-// output columns of its token: each valid (token, slot) row is written ONCE, in bf16, as whole 128-byte lines, to
-// y[slot]: top_k result rows per token instead of the top_k * I/128 partial rows the reference's decomposition
+// Down projection.  64 output columns at a time (4 operand tiles of w2 rows through the pair's ring), all slices,
+// the wavefront's token half.  The w2 rows of a tile are picked so that a lane ends up with 16 adjacent output columns
+// of its token: each valid (token, slot) row is written ONCE, in bf16, as whole 128-byte lines, to y[slot]: top_k
+// result rows per token instead of the top_k * I/128 partial rows the reference's decomposition
 // (fused_moe_w8a8_up_down_acc.cu:676-679,1085-1091) adds into the output.  A second kernel sums a token's live rows
 // in fp32 and rounds into `out` once.  No atomics: at M = 8192 fp32 atomics alone cost 13 ms on MI355X.
 //
@@ -45,6 +53,19 @@ struct TileParams {
     uint8_t *aqs;     // [row blocks][n_ib][TM] requantised operand tiles of 2 KiB
     int n_ib, nkb, n_mb_max;
 };
+
+#ifdef ALPHA_MOE_TRACE
+// Debug builds only: 100 MHz wall-clock stamps of wavefront 0 per up/gate step: loads landed, barrier passed, next
+// loads issued, step computed.
+// Stamps are kept in LDS during the kernel (a global store would join the vector-memory queue that the step
+// loop counts) and written out at the end.
+constexpr int kTraceSteps = 112;
+__device__ unsigned int g_tile_trace[1024][kTraceSteps][4];
+#define TILE_STAMP(step, i)                                                                       \
+    if (tid == 0 && (step) < kTraceSteps) s_trace[step][i] = (unsigned int)wall_clock64()
+#else
+#define TILE_STAMP(step, i)
+#endif
 
 typedef const void __attribute__((address_space(1))) * gptr_t;
 typedef void __attribute__((address_space(3))) * lptr_t;
@@ -76,13 +97,16 @@ __device__ __forceinline__ void lds_barrier()
     __builtin_amdgcn_sched_barrier(0);
 }
 
-// One step of a wavefront: 4 weight tiles x TM token tiles, all from LDS.  acc[k][t] += (A_k x B_t) * row[t] * sc[k & 1]
+// One step of a wavefront: 4 weight tiles x TH token tiles, all from LDS.  acc[k][t] += (A_k x B_t) * row[t] * sc[k & 1]
 // with row[] a per-token factor in LDS (16 floats per tile, already offset to this lane's token).  The product of
 // (k, t) is scaled into its accumulator behind the matrix instruction of (k, t + 1).
-template <int TM>
+// The step's NOPS direct-to-LDS loads (issue(i), i < NOPS) are spread evenly between the 4 TH matrix instructions: a
+// load instruction blocks its wavefront for 30-60 ns (measured), and the other wavefront of the SIMD computes then.
+template <int TH, int NOPS, typename Issue>
 __device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *b_tiles, const float *row, float sc0,
-                                         float sc1, v4f (&acc)[4][TM], int frag_lo, int frag_hi)
+                                         float sc1, v4f (&acc)[4][TH], int frag_lo, int frag_hi, Issue issue)
 {
+    constexpr int GROUPS = 4 * TH;
     auto read_tile = [&](const uint8_t *tile) -> v8i {
         return cat(*reinterpret_cast<const v4i *>(tile + frag_lo), *reinterpret_cast<const v4i *>(tile + frag_hi));
     };
@@ -94,10 +118,10 @@ __device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *
     v4f prev[4];
     float p0 = 0.f, p1 = 0.f;
 #pragma unroll
-    for (int t = 0; t < TM; t++) {
+    for (int t = 0; t < TH; t++) {
         v8i b_next = b;
         float f_next = f;
-        if (t + 1 < TM) {
+        if (t + 1 < TH) {
             b_next = read_tile(b_tiles + (t + 1) * 2048);
             f_next = row[(t + 1) * 16];
         }
@@ -105,7 +129,15 @@ __device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             cur[k] = mfma_fp8(a[k], b);
-            if (t > 0) acc[k][t - 1] += prev[k] * ((k & 1) ? p1 : p0);
+            if (t > 0) {
+                acc[k][t - 1] += prev[k] * ((k & 1) ? p1 : p0);
+                asm volatile("" : "+v"(acc[k][t - 1]));   // the multiply-adds stay here, behind this matrix instruction
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            // loads i with i * GROUPS / NOPS == g go behind group g
+#pragma unroll
+            for (int i = 0; i < NOPS; i++)
+                if (i * GROUPS / NOPS == t * 4 + k) issue(i);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -116,20 +148,21 @@ __device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *
         f = f_next;
     }
 #pragma unroll
-    for (int k = 0; k < 4; k++) acc[k][TM - 1] += prev[k] * ((k & 1) ? p1 : p0);
+    for (int k = 0; k < 4; k++) acc[k][TH - 1] += prev[k] * ((k & 1) ? p1 : p0);
 }
 
-// TM: 16-token tiles per row block.
-template <int TM>
-__global__ __launch_bounds__(256) void moe_tile_kernel(const TileParams s)
+// TH: 16-token tiles per wavefront; a row block has TM = 2 TH of them (block_m rounded up to 32 rows).
+// Wavefront v = (w = v % 4, g = v / 4): weight rows 64 w .. 64 w + 63 of the slice, token tiles g TH .. g TH + TH - 1.
+template <int TH>
+__global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
 {
-    constexpr int THREADS = 256;
-    constexpr int XT = (TM + 3) / 4;          // token tiles each wavefront gathers per K block
-    constexpr int XOPS = 3 * XT;              // its vector-memory operations for that: 2 tile halves + 16 scales
-    constexpr int AOPS = 8;                   // 4 weight tiles x 2 halves
+    constexpr int TM = 2 * TH;
+    constexpr int THREADS = 512;
+    constexpr int AOPS = 4;                   // 2 of the pair's 4 weight tiles x 2 halves
+    constexpr int XOPS = 3;                   // one token tile (2 halves) + its 16 scales
     constexpr int OPS1 = AOPS + XOPS;
 
-    // [4 wavefronts][3 stages][4 tiles] weight rings | [3 stages][TM] token tiles; the requantised tiles [n_ib][TM]
+    // [4 pairs][3 stages][4 tiles] weight rings | [3 stages][TM] token tiles; the requantised tiles [n_ib][TM]
     // later take the place of the token tiles
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds_dyn[];
     __shared__ __attribute__((aligned(1024))) uint8_t s_dummy[2048 + 64];
@@ -139,6 +172,9 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const TileParams s)
     __shared__ float s_sa[kTileMaxIb][TM * 16];
     __shared__ float s_w2s[kTileMaxW2s];
     __shared__ int s_tok[TM * 16];
+#ifdef ALPHA_MOE_TRACE
+    __shared__ unsigned int s_trace[kTraceSteps][4];
+#endif
 
     const MoeParams &p = s.p;
     // consecutive row blocks on one XCD: workgroup i runs on XCD i % 8
@@ -153,12 +189,13 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const TileParams s)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int w = wave & 3, g = wave >> 2;
     const int n = lane & 15;
     const int q = lane >> 4;
     const int K = p.K, I = p.N >> 1;
     const int n_ib = s.n_ib, nkb = s.nkb;
     const int epoch = __builtin_amdgcn_readfirstlane(s.ctl->epoch) + 1;
-    uint8_t *a_ring = lds_dyn + wave * (kStages * 8192);
+    uint8_t *a_ring = lds_dyn + w * (kStages * 8192);
     uint8_t *xbuf = lds_dyn + kARingBytes;
 
     // operand fragment of lane (n, q): chunks q and q+4 of row n; chunk c of row r sits at position c ^ ((r >> 1) & 7)
@@ -172,17 +209,17 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const TileParams s)
     for (int h = 0; h < 2; h++) ld_chunk[h] = 16 * ((lane & 7) ^ (((8 * h + ld_row) >> 1) & 7));
 
     // ---- routing ---------------------------------------------------------------------------------------------
-    int slot[TM];
-    bool valid[TM];
+    int slot[TH];
+    bool valid[TH];
 #pragma unroll
-    for (int t = 0; t < TM; t++) {
-        const int row = t * 16 + n;
+    for (int t = 0; t < TH; t++) {
+        const int row = (g * TH + t) * 16 + n;
         const int idx = mb * p.block_m + row;
         int id = -1;
         if (row < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
         valid[t] = id >= 0 && id / p.top_k < p.M;
         slot[t] = valid[t] ? id : 0;
-        if (wave == 0 && q == 0 && valid[t]) s.live[slot[t]] = epoch;
+        if (w == 0 && q == 0 && valid[t]) s.live[slot[t]] = epoch;
     }
     if (tid < TM * 16) {
         const int idx = mb * p.block_m + tid;
@@ -194,78 +231,75 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const TileParams s)
     for (int i = tid; i < (K >> 7) * n_ib; i += THREADS) s_w2s[i] = p.w2_scale[(size_t)e * (K >> 7) * n_ib + i];
     __syncthreads();
 
-    // token-tile gather: wavefront w loads tiles w and w+4 (a dummy where the block has no such tile)
-    const uint8_t *gx[XT][2];
-    const float *gxs[XT];
-    int xdst[XT];       // byte offset of the tile inside a ring stage, or -1: dummy
+    // token-tile gather: wavefront v loads tile v (a dummy where the block has no such tile)
+    const bool x_real = wave < TM;
+    const uint8_t *gx[2];
 #pragma unroll
-    for (int k = 0; k < XT; k++) {
-        const int t = wave + 4 * k;
-        const bool real = t < TM;
-        xdst[k] = real ? t * 2048 : -1;
-#pragma unroll
-        for (int h = 0; h < 2; h++)
-            gx[k][h] = p.x + (size_t)s_tok[real ? t * 16 + 8 * h + ld_row : 0] * K + ld_chunk[h];
-        gxs[k] = p.x_scale + (size_t)s_tok[real ? t * 16 + (lane & 15) : 0] * nkb;
-    }
-    auto issue_x = [&](int kb, int stage) {   // XOPS operations
+    for (int h = 0; h < 2; h++) gx[h] = p.x + (size_t)s_tok[x_real ? wave * 16 + 8 * h + ld_row : 0] * K + ld_chunk[h];
+    const float *gxs = p.x_scale + (size_t)s_tok[x_real ? wave * 16 + (lane & 15) : 0] * nkb;
+    auto issue_x_op = [&](int kb, int stage, int part) {   // operation `part` of XOPS
         const int kc = kb < nkb ? kb : nkb - 1;
-#pragma unroll
-        for (int k = 0; k < XT; k++) {
-            uint8_t *dst = xdst[k] >= 0 ? xbuf + stage * (TM * 2048) + xdst[k] : s_dummy;
-            dma16(gx[k][0] + (size_t)kc * 128, dst);
-            dma16(gx[k][1] + (size_t)kc * 128, dst + 1024);
-            float *sdst = xdst[k] >= 0 ? &s_xs[stage][(wave + 4 * k) * 16] : reinterpret_cast<float *>(s_dummy + 2048);
-            if (lane < 16) dma4(gxs[k] + kc, sdst);
+        if (part < 2) {
+            uint8_t *dst = x_real ? xbuf + stage * (TM * 2048) + wave * 2048 : s_dummy;
+            dma16(gx[part] + (size_t)kc * 128, dst + part * 1024);
+        } else {
+            float *sdst = x_real ? &s_xs[stage][wave * 16] : reinterpret_cast<float *>(s_dummy + 2048);
+            if (lane < 16) dma4(gxs + kc, sdst);
         }
     };
 
-    v4f acc[4][TM];
+    v4f acc[4][TH];
     for (int ib = 0; ib < n_ib; ib++) {
         // this slice's gate (row 2*ib) and up (row 2*ib+1) scale rows
         {
             const float *ws_rows = p.w_scale + ((size_t)e * (p.N >> 7) + 2 * ib) * nkb;
             for (int i = tid; i < 2 * nkb; i += THREADS) s_ws[i >= nkb][i >= nkb ? i - nkb : i] = ws_rows[i];
         }
-        // Weight rows of this wavefront: tile a = (pair a / 2, gate | up a % 2); matrix row r of the tile is slab row
-        // pair * 32 + (r / 8) * 16 + r % 8 (+ 8 for up), so load h of a tile covers slab rows ... + 16 h + lane / 8.
-        const uint8_t *wbase = p.w + ((size_t)e * p.N + ib * 256 + wave * 64 + ld_row) * K;
-        auto issue_a = [&](int kb, int stage) {   // AOPS operations
-            const int kc = kb < nkb ? kb : nkb - 1;
-            uint8_t *dst = a_ring + stage * 8192;
+        // Weight rows of the pair: tile a = (32-row group a / 2, gate | up a % 2); matrix row r of the tile is slab row
+        // group * 32 + (r / 8) * 16 + r % 8 (+ 8 for up), so load h of a tile covers slab rows ... + 16 h + lane / 8.
+        // Wavefront (w, g) loads tiles 2g and 2g + 1 of pair w.
+        const uint8_t *wbase = p.w + ((size_t)e * p.N + ib * 256 + w * 64 + g * 32 + ld_row) * K;
+        // operation i of a step's OPS1: weight tile half (i < AOPS) or a token-tile operation
+        auto issue_op = [&](int kb, int stage, int i) {
+            if (i < AOPS) {
+                const int kc = kb < nkb ? kb : nkb - 1;
+                const int up = i >> 1, h = i & 1;
+                dma16(wbase + (size_t)(h * 16 + 8 * up) * K + (size_t)kc * 128 + ld_chunk[h],
+                      a_ring + stage * 8192 + (2 * g + up) * 2048 + h * 1024);
+            } else {
+                issue_x_op(kb, stage, i - AOPS);
+            }
+        };
+        auto issue_all = [&](int kb, int stage) {
 #pragma unroll
-            for (int a = 0; a < 4; a++)
-#pragma unroll
-                for (int h = 0; h < 2; h++)
-                    dma16(wbase + (size_t)((a >> 1) * 32 + h * 16 + 8 * (a & 1)) * K + (size_t)kc * 128 + ld_chunk[h],
-                          dst + a * 2048 + h * 1024);
+            for (int i = 0; i < OPS1; i++) issue_op(kb, stage, i);
         };
 #pragma unroll
         for (int a = 0; a < 4; a++)
 #pragma unroll
-            for (int t = 0; t < TM; t++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+            for (int t = 0; t < TH; t++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
 
         // Per wavefront the loads of step kb are issued two steps ahead.  Step kb: wait for the own loads of kb (those of
-        // kb + 1 stay in flight), meet the others (their token tiles of kb have landed, and everybody is done reading
-        // stage (kb + 2) % 3), refill that stage, compute.
+        // kb + 1 stay in flight), meet the others (their tiles of kb have landed, and everybody is done reading
+        // stage (kb + 2) % 3), then compute while refilling that stage.
         __syncthreads();   // s_ws written; everybody is done with the previous slice
-        issue_a(0, 0);
-        issue_x(0, 0);
-        issue_a(1, 1);
-        issue_x(1, 1);
+        issue_all(0, 0);
+        issue_all(1, 1);
         for (int kb0 = 0; kb0 < nkb; kb0 += kStages) {
 #pragma unroll
             for (int h = 0; h < kStages; h++) {
                 const int kb = kb0 + h;
                 if (kb < nkb) {
                     wait_vmcnt<OPS1>();
+                    TILE_STAMP(ib * nkb + kb, 0);
                     lds_barrier();
-                    issue_a(kb + 2, (h + 2) % kStages);
-                    issue_x(kb + 2, (h + 2) % kStages);
+                    TILE_STAMP(ib * nkb + kb, 1);
+                    TILE_STAMP(ib * nkb + kb, 2);
+                    mma_step<TH, OPS1>(a_ring + h * 8192, xbuf + h * (TM * 2048) + g * (TH * 2048),
+                                       &s_xs[h][g * (TH * 16) + n], s_ws[0][kb], s_ws[1][kb], acc, frag_lo, frag_hi,
+                                       [&](int i) { issue_op(kb + 2, (h + 2) % kStages, i); });
                     __builtin_amdgcn_sched_barrier(0);
-                    mma_step<TM>(a_ring + h * 8192, xbuf + h * (TM * 2048), &s_xs[h][n], s_ws[0][kb], s_ws[1][kb], acc,
-                                 frag_lo, frag_hi);
-                    __builtin_amdgcn_sched_barrier(0);
+                    TILE_STAMP(ib * nkb + kb, 3);
                 }
             }
         }
@@ -273,7 +307,7 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const TileParams s)
 
         // ---- SwiGLU, per-token amax over the slice's 128 columns, FP8 requant into operand tiles (scratch) ---------
 #pragma unroll
-        for (int t = 0; t < TM; t++) {
+        for (int t = 0; t < TH; t++) {
             float m = 0.f;
 #pragma unroll
             for (int pr = 0; pr < 2; pr++)
@@ -285,31 +319,36 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const TileParams s)
                 }
             m = fmaxf(m, __shfl_xor(m, 16));
             m = fmaxf(m, __shfl_xor(m, 32));
-            if (q == 0) s_amax[wave][t * 16 + n] = m;
+            if (q == 0) s_amax[w][(g * TH + t) * 16 + n] = m;
         }
         __syncthreads();
 #pragma unroll
-        for (int t = 0; t < TM; t++) {
+        for (int t = 0; t < TH; t++) {
+            const int tg = g * TH + t;
             float m = kAmaxFloor;
 #pragma unroll
-            for (int wv = 0; wv < 4; wv++) m = fmaxf(m, s_amax[wv][t * 16 + n]);
+            for (int wv = 0; wv < 4; wv++) m = fmaxf(m, s_amax[wv][tg * 16 + n]);
             const float s_a = m / kFp8Max;
-            uint8_t *tile = s.aqs + ((size_t)(mb * n_ib + ib) * TM + t) * 2048;
+            uint8_t *tile = s.aqs + ((size_t)(mb * n_ib + ib) * TM + tg) * 2048;
 #pragma unroll
             for (int pr = 0; pr < 2; pr++) {
                 const uint32_t packed =
                     pack_fp8x4(clamp_fp8(acc[2 * pr][t][0] / s_a), clamp_fp8(acc[2 * pr][t][1] / s_a),
                                clamp_fp8(acc[2 * pr][t][2] / s_a), clamp_fp8(acc[2 * pr][t][3] / s_a));
-                // columns wave*32 + pr*16 + 4q .. +3 of token n: chunk wave*2 + pr of the row, bytes 4q .. 4q+3 in it
-                *reinterpret_cast<uint32_t *>(tile + n * 128 + 16 * ((wave * 2 + pr) ^ f_n) + 4 * q) = packed;
+                // columns w*32 + pr*16 + 4q .. +3 of token n: chunk w*2 + pr of the row, bytes 4q .. 4q+3 in it
+                *reinterpret_cast<uint32_t *>(tile + n * 128 + 16 * ((w * 2 + pr) ^ f_n) + 4 * q) = packed;
             }
-            if (wave == 0 && q == 0) s_sa[ib][t * 16 + n] = s_a;
+            if (w == 0 && q == 0) s_sa[ib][tg * 16 + n] = s_a;
         }
     }
     // the requantised tiles come back from scratch (L2) into LDS where the token ring was
     __syncthreads();   // also waits for this wavefront's scratch stores
+#ifdef ALPHA_MOE_TRACE
+    if (blockIdx.x < 1024)
+        for (int i = tid; i < kTraceSteps * 4; i += THREADS) (&g_tile_trace[blockIdx.x][0][0])[i] = (&s_trace[0][0])[i];
+#endif
     uint8_t *aq = xbuf;
-    for (int i = wave; i < n_ib * TM; i += 4) {
+    for (int i = wave; i < n_ib * TM; i += 8) {
         const uint8_t *src = s.aqs + ((size_t)mb * n_ib * TM + i) * 2048 + lane * 16;
         dma16(src, aq + i * 2048);
         dma16(src + 1024, aq + i * 2048 + 1024);
@@ -318,80 +357,85 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const TileParams s)
     __syncthreads();
 
     // ---- down projection: 64 output columns per step group, all slices ---------------------------------------------
-    // Matrix row r of tile k is output column c0 + 16 (r / 4) + 4 k + r % 4, so lane (n, q) collects columns
-    // c0 + 16 q .. c0 + 16 q + 15 of token n over the four tiles.  Load h of a tile: rows 8h + lane / 8.
-    float tw[TM];
+    // Pair w takes column groups w, w + 4, ...; its two wavefronts split the tokens as before and each loads two of the
+    // four w2 tiles of a step.  Matrix row r of tile k is output column c0 + 16 (r / 4) + 4 k + r % 4, so lane (n, q)
+    // collects columns c0 + 16 q .. c0 + 16 q + 15 of token n over the four tiles.  Load h of a tile: rows 8h + lane / 8.
+    float tw[TH];
 #pragma unroll
-    for (int t = 0; t < TM; t++) tw[t] = valid[t] ? p.topk_w[slot[t]] * p.scaling : 0.f;
+    for (int t = 0; t < TH; t++) tw[t] = valid[t] ? p.topk_w[slot[t]] * p.scaling : 0.f;
     const int n_groups = K >> 6;
-    const int my_groups = (n_groups - wave + 3) >> 2;   // column groups wave, wave + 4, ...
-    const int n_steps = my_groups * n_ib;               // (group, slice) steps, slice-minor
+    const int my_groups = (n_groups - w + 3) >> 2;            // column groups w, w + 4, ...
+    const int n_steps = ((n_groups + 3) >> 2) * n_ib;         // (group, slice) steps of the longest pair, slice-minor
     const uint8_t *w2base = p.w2 + ((size_t)e * K + 16 * (lane >> 5) + (ld_row & 3)) * I;
     int lg = 0, lib = 0;   // (group index, slice) of the next step to load
-    auto issue2 = [&](int stage) {   // AOPS operations
+    auto issue2_op = [&](int stage, int i) {   // operation i of AOPS of the step (lg, lib)
         const int gc = lg < my_groups ? lg : my_groups - 1;
-        const int c0 = (wave + 4 * gc) << 6;
-        uint8_t *dst = a_ring + stage * 8192;
-#pragma unroll
-        for (int k = 0; k < 4; k++)
-#pragma unroll
-            for (int h = 0; h < 2; h++)
-                dma16(w2base + (size_t)(c0 + 32 * h + 4 * k) * I + lib * 128 + ld_chunk[h], dst + k * 2048 + h * 1024);
+        const int c0 = (w + 4 * gc) << 6;
+        const int k = 2 * g + (i >> 1), h = i & 1;
+        dma16(w2base + (size_t)(c0 + 32 * h + 4 * k) * I + lib * 128 + ld_chunk[h],
+              a_ring + stage * 8192 + k * 2048 + h * 1024);
+    };
+    auto advance2 = [&]() {
         lib++;
         if (lib == n_ib) {
             lib = 0;
             lg++;
         }
     };
+    auto issue2 = [&](int stage) {
+#pragma unroll
+        for (int i = 0; i < AOPS; i++) issue2_op(stage, i);
+        advance2();
+    };
 #pragma unroll
     for (int a = 0; a < 4; a++)
 #pragma unroll
-        for (int t = 0; t < TM; t++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < TH; t++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
     int cg = 0, cib = 0;
-    if (n_steps > 0) {
-        issue2(0);
-        issue2(1);
-        for (int s0 = 0; s0 < n_steps; s0 += kStages) {
+    issue2(0);
+    issue2(1);
+    for (int s0 = 0; s0 < n_steps; s0 += kStages) {
 #pragma unroll
-            for (int h = 0; h < kStages; h++) {
-                if (s0 + h < n_steps) {
-                    // one younger step of AOPS loads stays in flight; result stores only make this stricter
-                    wait_vmcnt<AOPS>();
-                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // done reading the stage that is refilled
-                    issue2((h + 2) % kStages);
-                    __builtin_amdgcn_sched_barrier(0);
-                    const int c0 = (wave + 4 * cg) << 6;
-                    const float ws2 = s_w2s[(c0 >> 7) * n_ib + cib];
-                    mma_step<TM>(a_ring + h * 8192, aq + cib * (TM * 2048), &s_sa[cib][n], ws2, ws2, acc, frag_lo, frag_hi);
-                    __builtin_amdgcn_sched_barrier(0);
-                    cib++;
-                    if (cib == n_ib) {
+        for (int h = 0; h < kStages; h++) {
+            if (s0 + h < n_steps) {
+                // one younger step of AOPS loads stays in flight; result stores only make this stricter
+                wait_vmcnt<AOPS>();
+                lds_barrier();
+                const int gcl = cg < my_groups ? cg : my_groups - 1;
+                const int c0 = (w + 4 * gcl) << 6;
+                const float ws2 = s_w2s[(c0 >> 7) * n_ib + cib];
+                mma_step<TH, AOPS>(a_ring + h * 8192, aq + cib * (TM * 2048) + g * (TH * 2048),
+                                   &s_sa[cib][g * (TH * 16) + n], ws2, ws2, acc, frag_lo, frag_hi,
+                                   [&](int i) { issue2_op((h + 2) % kStages, i); });
+                advance2();
+                __builtin_amdgcn_sched_barrier(0);
+                cib++;
+                if (cib == n_ib) {
 #pragma unroll
-                        for (int t = 0; t < TM; t++) {
-                            if (valid[t]) {
-                                uint16_t *yp = s.y + (size_t)slot[t] * K + c0 + 16 * q;
+                    for (int t = 0; t < TH; t++) {
+                        if (valid[t] && cg < my_groups) {
+                            uint16_t *yp = s.y + (size_t)slot[t] * K + c0 + 16 * q;
 #pragma unroll
-                                for (int half = 0; half < 2; half++) {
-                                    const v4f lo = acc[2 * half][t] * tw[t], hi = acc[2 * half + 1][t] * tw[t];
-                                    v4i o;
-                                    o.x = (int)pack_bf16x2(lo[0], lo[1]);
-                                    o.y = (int)pack_bf16x2(lo[2], lo[3]);
-                                    o.z = (int)pack_bf16x2(hi[0], hi[1]);
-                                    o.w = (int)pack_bf16x2(hi[2], hi[3]);
-                                    *reinterpret_cast<v4i *>(yp + 8 * half) = o;
-                                }
+                            for (int half = 0; half < 2; half++) {
+                                const v4f lo = acc[2 * half][t] * tw[t], hi = acc[2 * half + 1][t] * tw[t];
+                                v4i o;
+                                o.x = (int)pack_bf16x2(lo[0], lo[1]);
+                                o.y = (int)pack_bf16x2(lo[2], lo[3]);
+                                o.z = (int)pack_bf16x2(hi[0], hi[1]);
+                                o.w = (int)pack_bf16x2(hi[2], hi[3]);
+                                *reinterpret_cast<v4i *>(yp + 8 * half) = o;
                             }
-#pragma unroll
-                            for (int a = 0; a < 4; a++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
                         }
-                        cib = 0;
-                        cg++;
+#pragma unroll
+                        for (int a = 0; a < 4; a++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
                     }
+                    cib = 0;
+                    cg++;
                 }
             }
         }
-        wait_vmcnt<0>();
     }
+    wait_vmcnt<0>();
 }
 
 // out[t] = bf16(out[t] + sum over the token's live slots of y[slot]); the last workgroup to leave closes the epoch.
@@ -451,17 +495,16 @@ int tail_tiles(int n_ib) { return n_ib > kStages ? n_ib : kStages; }
 
 typedef void (*TileFn)(const TileParams);
 
-TileFn pick(int tm)
+// 16-token tiles per wavefront: a row block is rounded up to 32 th rows
+int tiles_per_wave(int block_m) { return (block_m + 31) / 32; }
+
+TileFn pick(int th)
 {
-    switch (tm) {
+    switch (th) {
     case 1: return moe_tile_kernel<1>;
     case 2: return moe_tile_kernel<2>;
     case 3: return moe_tile_kernel<3>;
-    case 4: return moe_tile_kernel<4>;
-    case 5: return moe_tile_kernel<5>;
-    case 6: return moe_tile_kernel<6>;
-    case 7: return moe_tile_kernel<7>;
-    default: return moe_tile_kernel<8>;
+    default: return moe_tile_kernel<4>;
     }
 }
 
@@ -471,7 +514,7 @@ bool tile_supported(int top_k, int M, int K, int N, int E, int sorted_num, int b
 {
     (void)E;
     (void)sorted_num;
-    const int tm = (block_m + 15) / 16;
+    const int tm = 2 * tiles_per_wave(block_m);
     const int n_ib = N / 256;
     return n_ib <= kTileMaxIb && tail_tiles(n_ib) * tm * 2048 <= kMaxTailBytes && K <= 128 * kTileMaxKb &&
            (K / 128) * n_ib <= kTileMaxW2s && (int64_t)M * top_k <= kMaxSlots;
@@ -480,7 +523,7 @@ bool tile_supported(int top_k, int M, int K, int N, int E, int sorted_num, int b
 size_t tile_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
 {
     (void)E;
-    const int tm = (block_m + 15) / 16;
+    const int tm = 2 * tiles_per_wave(block_m);
     const size_t n_mb = ((size_t)sorted_num + block_m - 1) / block_m;
     return align_up(kPrefixBytes) + align_up((size_t)M * top_k * K * sizeof(uint16_t)) +
            align_up(n_mb * (N / 256) * tm * 2048);
@@ -498,14 +541,14 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
     s.n_ib = p.N / 256;
     s.nkb = p.K / 128;
     s.n_mb_max = (p.sorted_num + p.block_m - 1) / p.block_m;
-    const int tm = (p.block_m + 15) / 16;
-    const TileFn fn = pick(tm);
+    const int tm = 2 * tiles_per_wave(p.block_m);
+    const TileFn fn = pick(tm / 2);
     const int lds_bytes = kARingBytes + tail_tiles(s.n_ib) * tm * 2048;
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          kARingBytes + kMaxTailBytes);
     if (err != hipSuccess) return err;
     const int grid = (s.n_mb_max + 7) / 8 * 8;
-    hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(256), lds_bytes, stream, s);
+    hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(512), lds_bytes, stream, s);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
     const int chunks = (p.K + 2047) / 2048;
@@ -516,3 +559,12 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
 }
 
 }  // namespace alpha_moe
+
+#ifdef ALPHA_MOE_TRACE
+extern "C" int alpha_moe_debug_tile_trace_read(void *dst)
+{
+    (void)hipDeviceSynchronize();
+    (void)hipMemcpyFromSymbol(dst, HIP_SYMBOL(alpha_moe::g_tile_trace), sizeof(alpha_moe::g_tile_trace));
+    return 1024 * alpha_moe::kTraceSteps;
+}
+#endif
