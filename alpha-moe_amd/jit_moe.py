@@ -11,7 +11,8 @@ Differences, all on purpose:
   * `--balancedness` is honoured (the reference parses it and then samples uniformly, jit_moe.py:135);
   * a call is timed with HIP events on the launch stream after a 512 MiB write that evicts L2 and the 256 MiB
     Infinity Cache (the reference allocates 2 GiB of randn before every call, jit_moe.py:21-22);
-  * `--block-ms`, `--stages` and `--num-tests` bound the sweep (the full space is 160 configurations);
+  * `--block-ms`, `--stages` and `--num-tests` bound the sweep (the full space is 160 configurations) and `--update`
+    merges the result into an existing table;
   * on MI355X `warp_n` counts 64-wide wavefronts per workgroup and `stages` sizes the LDS ring.
 """
 import argparse
@@ -75,6 +76,8 @@ def parse_arguments(argv=None):
     parser.add_argument("--block-ms", type=int, nargs="+", default=list(range(8, 129, 8)), help="block_m values to sweep")
     parser.add_argument("--stages", type=int, nargs="+", default=[1, 2, 3, 4, 5], help="stages values to sweep")
     parser.add_argument("--num-tests", type=int, default=25, help="timed calls per configuration and routing sample")
+    parser.add_argument("--update", action="store_true",
+                        help="keep the entries --out-config already holds for batch sizes not benchmarked in this run")
     return parser.parse_args(argv)
 
 
@@ -126,6 +129,11 @@ def main(argv=None):
         conf_to_save[nt] = {"block_m": block_m, "block_n": bn, "warp_n": wn, "stages": stages}
 
     out_config = args.out_config or f"moe_jit_{E}_{N}_{K}.json"
+    if args.update and os.path.exists(out_config):
+        with open(out_config) as f:
+            merged = {int(k): v for k, v in json.load(f).items()}
+        merged.update(conf_to_save)
+        conf_to_save = dict(sorted(merged.items()))
     with open(out_config, "w") as f:
         json.dump(conf_to_save, f)
     return 0
