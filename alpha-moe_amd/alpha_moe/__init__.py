@@ -1,5 +1,6 @@
 """``import alpha_moe`` registers ``torch.ops.alpha_moe.fused_moe_w8a8_up_down`` (as the reference's extension
-module of the same name does, csrc/torch_interface.cpp:105-131) by loading the in-tree HIP libraries.
+module of the same name does, csrc/torch_interface.cpp:105-131) by loading the in-tree HIP libraries, together with
+the two input-preparation operators ``per_token_group_quant_fp8`` and ``moe_align_block_size``.
 
 There is no fallback: if the libraries are not built the import fails.
 """
@@ -30,5 +31,15 @@ c_abi.alpha_moe_fused_moe_w8a8_up_down.argtypes = (
     [ctypes.c_void_p] * 11 + [ctypes.c_int] * 10 + [ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p])
 c_abi.alpha_moe_workspace_bytes.restype = ctypes.c_size_t
 c_abi.alpha_moe_workspace_bytes.argtypes = [ctypes.c_int] * 7
+
+c_abi.alpha_moe_per_token_group_quant_fp8.restype = ctypes.c_int
+c_abi.alpha_moe_per_token_group_quant_fp8.argtypes = (
+    [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p])
+c_abi.alpha_moe_align_workspace_bytes.restype = ctypes.c_size_t
+c_abi.alpha_moe_align_workspace_bytes.argtypes = [ctypes.c_int] * 2
+c_abi.alpha_moe_moe_align_block_size.restype = ctypes.c_int
+c_abi.alpha_moe_moe_align_block_size.argtypes = (
+    [ctypes.c_void_p] + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,
+                                              ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p])
 
 __version__ = c_abi.alpha_moe_version().decode()

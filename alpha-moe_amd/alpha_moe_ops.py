@@ -15,6 +15,19 @@ def _fused_moe_w8a8_up_down_fake(x, x_scale, w, w_scale, w2, w2_scale, sorted_to
     return None
 
 
+@torch.library.register_fake("alpha_moe::per_token_group_quant_fp8")
+def _per_token_group_quant_fp8_fake(x, group_size):
+    return (torch.empty_like(x, dtype=torch.float8_e4m3fn),
+            x.new_empty((x.shape[0], x.shape[1] // group_size), dtype=torch.float32))
+
+
+@torch.library.register_fake("alpha_moe::moe_align_block_size")
+def _moe_align_block_size_fake(topk_ids, block_size, num_experts):
+    sorted_num = topk_ids.numel() + num_experts * (block_size - 1)
+    return (topk_ids.new_empty((sorted_num,)), topk_ids.new_empty(((sorted_num + block_size - 1) // block_size,)),
+            topk_ids.new_empty((1,)))
+
+
 def fused_moe_w8a8_up_down(
     x: torch.Tensor,
     x_scale: torch.Tensor,

@@ -15,6 +15,7 @@
 #include "../../include/alpha_moe_hip.h"
 
 #include <map>
+#include <tuple>
 #include <mutex>
 #include <utility>
 
@@ -111,10 +112,63 @@ void fused_moe_w8a8_up_down(const at::Tensor &x, const at::Tensor &x_scale, cons
     TORCH_CHECK(rc == ALPHA_MOE_OK, "alpha_moe_fused_moe_w8a8_up_down failed: ", alpha_moe_status_string(rc));
 }
 
+// (q, scale) = per_token_group_quant_fp8(x, 128): what the reference's callers get from SGLang (jit_moe.py:142).
+std::tuple<at::Tensor, at::Tensor> per_token_group_quant_fp8(const at::Tensor &x, int64_t group_size)
+{
+    TORCH_CHECK(x.is_cuda(), "x must be a GPU tensor");
+    TORCH_CHECK(group_size == 128, "group_size must be 128");
+    TORCH_CHECK(x.dim() == 2 && x.size(1) % 128 == 0 && x.size(0) > 0, "x must be [M, K] with K % 128 == 0");
+    TORCH_CHECK(x.scalar_type() == at::kBFloat16 || x.scalar_type() == at::kFloat, "x must be bfloat16 or float32");
+    TORCH_CHECK(x.is_contiguous(), "x must be contiguous");
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(x.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    at::Tensor q = at::empty(x.sizes(), x.options().dtype(at::kFloat8_e4m3fn));
+    at::Tensor scale = at::empty({x.size(0), x.size(1) / 128}, x.options().dtype(at::kFloat));
+    const int rc = alpha_moe_per_token_group_quant_fp8(x.const_data_ptr(), x.scalar_type() == at::kFloat,
+                                                       static_cast<uint8_t *>(q.data_ptr()), scale.data_ptr<float>(),
+                                                       static_cast<int>(x.size(0)), static_cast<int>(x.size(1)),
+                                                       static_cast<void *>(stream));
+    TORCH_CHECK(rc == ALPHA_MOE_OK, "alpha_moe_per_token_group_quant_fp8 failed: ", alpha_moe_status_string(rc));
+    return {q, scale};
+}
+
+// (sorted_token_ids, expert_ids, num_tokens_post_padded) = moe_align_block_size(topk_ids, block_size, num_experts):
+// what the reference's callers get from SGLang (jit_moe.py:158).
+std::tuple<at::Tensor, at::Tensor, at::Tensor> moe_align_block_size(const at::Tensor &topk_ids, int64_t block_size,
+                                                                    int64_t num_experts)
+{
+    TORCH_CHECK(topk_ids.is_cuda(), "topk_ids must be a GPU tensor");
+    TORCH_CHECK(topk_ids.scalar_type() == at::kInt, "topk_ids must be int32");
+    TORCH_CHECK(topk_ids.is_contiguous() && topk_ids.numel() > 0, "topk_ids must be contiguous and not empty");
+    TORCH_CHECK(block_size > 0 && num_experts > 0, "block_size and num_experts must be positive");
+    const int64_t numel = topk_ids.numel();
+    const int64_t sorted_num = numel + num_experts * (block_size - 1);
+    const int64_t n_blocks = (sorted_num + block_size - 1) / block_size;
+    TORCH_CHECK(sorted_num <= INT32_MAX, "too many routing slots");
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA guard(topk_ids.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    const auto opts = topk_ids.options();
+    at::Tensor sorted_ids = at::empty({sorted_num}, opts), expert_ids = at::empty({n_blocks}, opts),
+               total = at::empty({1}, opts);
+    const size_t ws_bytes = alpha_moe_align_workspace_bytes(static_cast<int>(numel), static_cast<int>(num_experts));
+    at::Tensor ws = at::empty({static_cast<int64_t>(ws_bytes)}, opts.dtype(at::kByte));
+    const int rc = alpha_moe_moe_align_block_size(
+        topk_ids.const_data_ptr<int32_t>(), static_cast<int>(numel), static_cast<int>(num_experts),
+        static_cast<int>(block_size), sorted_ids.data_ptr<int32_t>(), static_cast<int>(sorted_num),
+        expert_ids.data_ptr<int32_t>(), static_cast<int>(n_blocks), total.data_ptr<int32_t>(), ws.data_ptr(), ws_bytes,
+        static_cast<void *>(stream));
+    TORCH_CHECK(rc == ALPHA_MOE_OK, "alpha_moe_moe_align_block_size failed: ", alpha_moe_status_string(rc));
+    return {sorted_ids, expert_ids, total};
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(alpha_moe, m)
 {
+    m.def("per_token_group_quant_fp8(Tensor x, int group_size) -> (Tensor, Tensor)");
+    m.impl("per_token_group_quant_fp8", c10::DispatchKey::CUDA, &per_token_group_quant_fp8);
+    m.def("moe_align_block_size(Tensor topk_ids, int block_size, int num_experts) -> (Tensor, Tensor, Tensor)");
+    m.impl("moe_align_block_size", c10::DispatchKey::CUDA, &moe_align_block_size);
     m.def("fused_moe_w8a8_up_down("
           "Tensor x, Tensor x_scale, Tensor w, Tensor w_scale, Tensor w2, Tensor w2_scale, "
           "Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_post_padded, Tensor topk_weights, "

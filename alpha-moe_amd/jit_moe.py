@@ -7,7 +7,7 @@ writer jit_moe.py:169-183):
     python alpha-moe_amd/jit_moe.py --E 256 --N 512 --K 7168 --out-config moe_jit_257_512_7168.json
 
 Differences, all on purpose:
-  * activations are quantised and routing arrays built by this package (alpha_moe_python.prep), not SGLang;
+  * activations are quantised and routing arrays built by this package's own HIP kernels (alpha_moe_python.prep_hip), not SGLang;
   * `--balancedness` is honoured (the reference parses it and then samples uniformly, jit_moe.py:135);
   * a call is timed with HIP events on the launch stream after a 512 MiB write that evicts L2 and the 256 MiB
     Infinity Cache (the reference allocates 2 GiB of randn before every call, jit_moe.py:21-22);
@@ -28,7 +28,7 @@ if HERE not in sys.path:
     sys.path.insert(0, HERE)
 
 import alpha_moe  # noqa: E402,F401  registers torch.ops.alpha_moe.fused_moe_w8a8_up_down
-from alpha_moe_python.prep import moe_align_block_size, per_token_group_quant_fp8  # noqa: E402
+from alpha_moe_python.prep_hip import moe_align_block_size, per_token_group_quant_fp8  # noqa: E402
 
 _FLUSH = None
 

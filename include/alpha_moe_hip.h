@@ -78,6 +78,35 @@ size_t alpha_moe_workspace_bytes(int top_k, int M, int K, int N, int num_experts
 int alpha_moe_validate(int top_k, int M, int K, int N, int num_experts, int sorted_num,
                        int block_m, int block_n, int warp_n, int stages);
 
+/*
+ * Input preparation, the two steps every caller runs right before the fused call.  The reference takes both from
+ * SGLang (jit_moe.py:142,158; extra/sglang.patch:30-35); here they are part of the library.
+ *
+ * alpha_moe_per_token_group_quant_fp8 replaces sglang_per_token_group_quant_fp8(x, 128) (jit_moe.py:142): x is
+ * [M, K] row-major bf16 (x_is_f32 == 0) or fp32 (x_is_f32 != 0), K % 128 == 0; writes q [M, K] FP8 e4m3 and
+ * scale [M, K/128] fp32 with scale = max(amax, 1e-10) / 448, q = rne(clamp(x / scale, -448, 448)): the arrays the
+ * fused kernel reads at fused_moe_w8a8_up_down_acc.cu:793,800-807.
+ */
+int alpha_moe_per_token_group_quant_fp8(const void *x, int x_is_f32, uint8_t *q, float *scale, int M, int K,
+                                        void *stream /* hipStream_t */);
+
+/*
+ * alpha_moe_moe_align_block_size replaces SGLang's moe_align_block_size(topk_ids, block_size, num_experts)
+ * (jit_moe.py:158): topk_ids holds the expert of each of the numel = M * top_k routing slots.  Writes
+ *   sorted_token_ids [sorted_num = numel + num_experts * (block_size - 1)]: slot ids in ascending expert order,
+ *       ascending within an expert, every expert's segment padded to a multiple of block_size with the value numel;
+ *   expert_ids [n_blocks = ceil(sorted_num / block_size)]: the expert of each block, -1 past the padded total;
+ *   num_tokens_post_padded [1]: the padded total
+ * as the fused kernel reads them (fused_moe_w8a8_up_down_acc.cu:676-679,756-758).  Slots whose expert is outside
+ * [0, num_experts) are dropped.  num_experts <= 4096.  Inputs of more than 4096 slots need a scratch buffer of
+ * alpha_moe_align_workspace_bytes(numel, num_experts) bytes (any contents); smaller ones accept workspace == NULL.
+ */
+size_t alpha_moe_align_workspace_bytes(int numel, int num_experts);
+int alpha_moe_moe_align_block_size(const int32_t *topk_ids, int numel, int num_experts, int block_size,
+                                   int32_t *sorted_token_ids, int sorted_num, int32_t *expert_ids, int n_blocks,
+                                   int32_t *num_tokens_post_padded, void *workspace, size_t workspace_bytes,
+                                   void *stream /* hipStream_t */);
+
 /* Human-readable text for a status code (static storage). */
 const char *alpha_moe_status_string(int status);
 

@@ -90,3 +90,26 @@ def test_workspace_bytes_is_monotone_and_covers_both_kernel_families(lib):
     direct = lib.alpha_moe_workspace_bytes(9, 64, 7168, 512, 257, 576 + 257 * 127, 128)
     assert direct >= 64 * 7168 * 4
     assert lib.alpha_moe_workspace_bytes(9, 0, 7168, 512, 257, 100, 16) == 0
+
+
+def test_prep_entry_points_refuse_bad_arguments_without_touching_a_device(lib):
+    lib.alpha_moe_per_token_group_quant_fp8.restype = ctypes.c_int
+    lib.alpha_moe_per_token_group_quant_fp8.argtypes = (
+        [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p])
+    lib.alpha_moe_align_workspace_bytes.restype = ctypes.c_size_t
+    lib.alpha_moe_align_workspace_bytes.argtypes = [ctypes.c_int] * 2
+    lib.alpha_moe_moe_align_block_size.restype = ctypes.c_int
+    lib.alpha_moe_moe_align_block_size.argtypes = (
+        [ctypes.c_void_p] + [ctypes.c_int] * 3 + [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,
+                                                  ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p])
+    assert lib.alpha_moe_per_token_group_quant_fp8(None, 0, None, None, 4, 128, None) == 1      # null pointer
+    assert lib.alpha_moe_per_token_group_quant_fp8(8, 0, 8, 8, 4, 130, None) == 2               # K % 128
+    assert lib.alpha_moe_align_workspace_bytes(0, 8) == 0
+    assert lib.alpha_moe_align_workspace_bytes(1024, 8) == 8 * 4
+    assert lib.alpha_moe_align_workspace_bytes(1025, 8) == 2 * 8 * 4
+    assert lib.alpha_moe_moe_align_block_size(None, 32, 8, 16, None, 0, None, 0, None, None, 0, None) == 1
+    # sorted_num must be numel + E * (block - 1), n_blocks its ceiling quotient
+    assert lib.alpha_moe_moe_align_block_size(8, 32, 8, 16, 8, 100, 8, 7, 8, None, 0, None) == 2
+    assert lib.alpha_moe_moe_align_block_size(8, 32, 5000, 16, 8, 32 + 5000 * 15, 8, 4690, 8, None, 0, None) == 2
+    # more than 4096 slots need the scratch buffer
+    assert lib.alpha_moe_moe_align_block_size(8, 5000, 8, 16, 8, 5120, 8, 320, 8, None, 0, None) == 7
