@@ -104,10 +104,12 @@ struct StreamCtl {
     int head;        // streaming kernel: next work item
     int done;        // streaming kernel: workgroups that have left
     int epoch;       // completed launches on this workspace (any kernel family)
-    int down_done;   // streaming kernel: finished DOWN items of this launch
     int error;       // sticky: a bounded wait ran out
     int fin_done;    // tile kernels: reduce-kernel workgroups that have left
-    int pad[58];
+    int pad0[27];
+    // a 128-byte line of its own: idle workgroups poll it while the others still fetch items through `head`
+    int down_done;   // streaming kernel: finished DOWN items of this launch
+    int pad1[31];
 };
 static_assert(sizeof(StreamCtl) == 256, "control block is one 256-byte line group");
 
