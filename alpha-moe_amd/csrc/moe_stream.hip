@@ -477,11 +477,16 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 }
             };
             int slot_w = 0, slot_r = 0;
+            auto prime = [&]() {
 #pragma unroll
-            for (int j = 0; j < S - 1; j++) {
-                issue(slot_w);
-                slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
-            }
+                for (int j = 0; j < S - 1; j++) {
+                    issue(slot_w);
+                    slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
+                }
+            };
+            // Wavefront 0 polls the flags, and a poll returns behind everything the wavefront has in flight: it fills its
+            // ring after the poll, the others before.
+            if (wave != 0) prime();
             // w2 scales of the 128-column blocks this item touches: s_sc[blk * n_ib + ib]
             const int blk0 = (t0 * 16) >> 7;
             const int nblk = (((t1 * 16) - 1) >> 7) - blk0 + 1;
@@ -493,6 +498,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 for (int ib = 0; ib < n_ib; ib++) spin_until_ge(&s.flag[mb * n_ib + ib], epoch, s.ctl);
             __syncthreads();
             TRACE_MARK;
+            if (wave == 0) prime();
 
             // requantised activations of all slices -> LDS as operand tiles, their scales -> s_xs[row][ib]
             for (int i = wave; i < n_ib * TM; i += WN) {
@@ -562,6 +568,9 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         TRACE_MARK;
         const int t = f / s.n_fc;
         const int c = (f - t * s.n_fc) * kFinCols + tid * 4;
+        // lane k fetches the stamp of the token's slot k: one round trip for all of them (top_k <= 64)
+        const int stamp = load_agent(&s.live[t * p.top_k + (lane < p.top_k ? lane : 0)]);
+        const unsigned long long live_mask = __ballot(lane < p.top_k && stamp == epoch);
         if (tid < kFinCols / 4 && c < K) {
             v4f sum = {0.f, 0.f, 0.f, 0.f};
             // slot order: the sum depends on nothing but the inputs.  Eight rows are in flight at a time.
@@ -570,7 +579,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
 #pragma unroll
                 for (int k = 0; k < 8; k++) {
                     const int slot = t * p.top_k + s0 + k;
-                    const bool on = s0 + k < p.top_k && load_agent(&s.live[slot]) == epoch;
+                    const bool on = s0 + k < p.top_k && ((live_mask >> (s0 + k)) & 1);
                     bits[k] = (v4i){0, 0, 0, 0};
                     if (on) bits[k] = ldg128_agent(s.y + (size_t)slot * K + c);
                 }
@@ -678,7 +687,7 @@ HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int bl
     if (n_mb_max > rows) n_mb_max = rows;
     h.n_mb_max = (int)n_mb_max;
     const int64_t units = n_mb_max * h.n_ib;
-    h.ok = block_m <= 32 && h.n_ib <= kMaxIb && units <= kMaxUnits && rows <= kMaxSlots &&
+    h.ok = block_m <= 32 && top_k <= 64 && h.n_ib <= kMaxIb && units <= kMaxUnits && rows <= kMaxSlots &&
            rows * (int64_t)K * 4 <= ((int64_t)1 << 30);
     if (!h.ok) return h;
     h.units = (int)units;
