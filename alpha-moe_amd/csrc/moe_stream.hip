@@ -674,6 +674,19 @@ struct HostPlan {
     size_t off_sa, off_aq, off_hpart, off_y, total;
 };
 
+// Compute units of the current device (256 on MI355X); read once.
+int compute_units()
+{
+    static const int n = [] {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            return 256;
+        return cus;
+    }();
+    return n;
+}
+
 HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
 {
     HostPlan h = {};
@@ -692,17 +705,18 @@ HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int bl
     if (!h.ok) return h;
     h.units = (int)units;
 
-    // Item sizes (from sweeps on MI355X, DeepSeek-V3 shard, M = 1..64): about one UP item per workgroup slot and
-    // K split, between 128 KiB and 1 MiB of w1 each - smaller items drown in their fixed cost (a dozen dependent
-    // memory round trips), larger ones leave a long tail; DOWN items of at most 256 KiB of w2.
-    const int slots = 512;
+    // Item sizes (from sweeps on MI355X, DeepSeek-V3 shard, M = 1..64).  UP: whole K per item once there are about as
+    // many (row block, slice) units as compute units - no partial sums, no arrival counter - and otherwise K split so
+    // that the UP items about fill the chip once; items below ~128 KiB of w1 drown in their fixed cost (a dozen
+    // dependent memory round trips).  DOWN: items of 256 KiB of w2, 128 KiB when there would be too few of them.
+    const int cus = compute_units();
     int64_t mb_est = (rows < E ? rows : E) + rows / block_m;
     if (mb_est > n_mb_max) mb_est = n_mb_max;
-    const int64_t unit_bytes = (int64_t)256 * K + (int64_t)K * 128;
-    int64_t target = mb_est * h.n_ib * unit_bytes / slots;
-    if (target < (128 << 10)) target = 128 << 10;
-    if (target > (1 << 20)) target = 1 << 20;
-    int kbpi = (int)((target + (1 << 14)) / (1 << 15));   // 32 KiB of w1 per K block
+    const int64_t units_est = mb_est * h.n_ib;
+    int ks_want = (int)((cus + units_est - 1) / units_est);
+    if (ks_want < 1) ks_want = 1;
+    int kbpi = (h.nkb + ks_want - 1) / ks_want;
+    if (kbpi < 4) kbpi = 4;
     kbpi = env_int("ALPHA_MOE_KBPI", kbpi);
     if (kbpi < 1) kbpi = 1;
     if (kbpi > h.nkb) kbpi = h.nkb;
@@ -711,7 +725,8 @@ HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int bl
     h.kbpi = (h.nkb + h.ks - 1) / h.ks;                    // even split
     h.ks = (h.nkb + h.kbpi - 1) / h.kbpi;
     // a DOWN item reads all n_ib slices of its columns: 2 KiB * n_ib per 16-column tile
-    const int64_t down_target = target < (256 << 10) ? target : (256 << 10);
+    int64_t down_target = 256 << 10;
+    if (mb_est * ((h.n_ct * 2048 * h.n_ib + down_target - 1) / down_target) < cus / 2) down_target = 128 << 10;
     int tpi = (int)(down_target / (2048 * h.n_ib)) / 16 * 16;
     tpi = env_int("ALPHA_MOE_TPI", tpi);
     if (tpi < 16) tpi = 16;
