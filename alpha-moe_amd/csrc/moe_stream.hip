@@ -121,13 +121,13 @@ __device__ __forceinline__ void store_agent(int *p, int v)
 }
 
 // Bounded wait for *addr >= target (one thread).  ~4M polls with a sleep between them, i.e. seconds.  The sleep grows
-// from 0.2 us to 0.9 us: a hundred workgroups polling one address every 0.2 us keep that L2 channel busy enough to
+// from 0.1 us to 0.9 us: a hundred workgroups polling one address every 0.2 us keep that L2 channel busy enough to
 // slow the loads of the workgroups still streaming weights threefold (measured).
 __device__ __noinline__ void spin_until_ge(const int *addr, int target, StreamCtl *ctl)
 {
     for (int it = 0; it < (1 << 22); it++) {
         if (load_agent(addr) >= target) return;
-        if (it < 4) __builtin_amdgcn_s_sleep(8);
+        if (it < 16) __builtin_amdgcn_s_sleep(4);
         else __builtin_amdgcn_s_sleep(32);
     }
     store_agent(&ctl->error, 1);
@@ -241,8 +241,10 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     // could already run.
     int next_item = -1;
     auto fetch_next = [&]() {
+        // the first gridDim.x items are handed out by workgroup index, the counter hands out the rest
         if (tid == 0 && next_item < 0)
-            next_item = __hip_atomic_fetch_add(&s.ctl->head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            next_item = (int)gridDim.x +
+                        __hip_atomic_fetch_add(&s.ctl->head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
 
     // SwiGLU + per-token amax over the 128 columns + FP8 requant of one unit, from accumulators in the MFMA layout.
@@ -631,9 +633,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         down_item(down);
         return 2;
     };
-    if (tid == 0) s_bcast[0] = __hip_atomic_fetch_add(&s.ctl->head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    int item = __builtin_amdgcn_readfirstlane(s_bcast[0]);
+    int item = blockIdx.x;   // no round trip to the queue before the first item
     while (item < total) {
         TRACE_BEGIN;
         next_item = -1;
