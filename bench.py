@@ -5,7 +5,9 @@
 
 A "step" is one call of torch.ops.alpha_moe.fused_moe_w8a8_up_down on a DeepSeek-V3-like single-GPU TP shard
 (E=257 incl. the fused shared expert, top_k=9, K=7168, I=256, FP8 e4m3 with 128x128 block scales) with all inputs
-resident in HBM.  The headline is M=64 decode; M = 1, 4, 16 are measured in the same run and reported under "per_M".
+resident in HBM.  The headline is M=64 decode against the HBM roofline; the same run also measures the other batch
+sizes of that shard (decode M = 1, 4, 16 and prefill M = 512, 2048, 8192, reported under "per_M" with both the HBM and
+the FP8 MFMA fraction) and the Qwen3-Next-like and Qwen3-30B-like shards ("other_configs").
 Consecutive steps rotate through several copies of the weights and several routings so that a step never finds its
 weights in the 256 MiB Infinity Cache; `out` is not re-zeroed inside the timed region (the operator adds into it).
 
@@ -26,10 +28,14 @@ sys.path.insert(0, ROOT)
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy of known size), for the
 # configurations that were profiled: profiles/moe_stream_kernel_ds_decode_M64_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES = {("ds", 64): 1302.5e6}
+#   profiles/moe_tile_kernel_ds_prefill_M8192_hbm_traffic.md (both kernels of a call)
+MEASURED_TRAFFIC_BYTES = {("ds", 64): 1296.3e6, ("ds", 8192): 5544.0e6}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
 DEFAULT_KNOBS = {"block_m": 16, "block_n": 32, "warp_n": 8, "stages": 5}
+# batch sizes of the other benchmark configurations
+DS_OTHER_M = (1, 4, 16, 64, 512, 2048, 8192)
+OTHER_CONFIGS = {"qn": (1, 32, 256, 4096), "q3": (64, 1024, 8192)}
 
 
 def parse_args():
@@ -40,6 +46,7 @@ def parse_args():
     ap.add_argument("--shape", default="ds", choices=["ds", "qn", "q3", "c1"])
     ap.add_argument("--M", type=int, default=64, help="tokens of the headline measurement")
     ap.add_argument("--also-M", type=int, nargs="*", default=None, help="other token counts reported under per_M")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the Qwen3-Next / Qwen3-30B shards")
     ap.add_argument("--replicas", type=int, default=6, help="copies of the weights rotated through")
     ap.add_argument("--config", default=None, help="tuning table (JSON of jit_moe.py); default: shipped table or built-in knobs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -66,61 +73,80 @@ def main():
 
     dev = "cuda:0"
     torch.cuda.set_device(0)
-    shape = SHAPES[args.shape]
-    cfg_path = args.config or os.path.join(ROOT, "alpha-moe_amd", "configs", f"moe_jit_{shape.E}_{shape.N}_{shape.K}.json")
-
-    def knobs_for(M):
-        if os.path.exists(cfg_path):
-            return dict(get_best_config(cfg_path, M)), os.path.relpath(cfg_path, ROOT)
-        return dict(DEFAULT_KNOBS), "built-in"
-
-    W0 = make_weights(shape, device=dev, seed=0)
-    replicas = [W0]
-    for _ in range(max(1, args.replicas) - 1):
-        replicas.append(Weights(shape, W0.w1.clone(), W0.w1_scale.clone(), W0.w2.clone(), W0.w2_scale.clone()))
     n_routings = 8
 
-    def prepare(M):
-        """Problems (routing + activations) for M tokens, one per routing seed, each bound to one weight replica."""
-        knobs, src = knobs_for(M)
-        calls, byts, flops = [], [], []
-        for i in range(n_routings):
-            W = replicas[i % len(replicas)]
-            P = make_problem(W, M, seed=i)
-            s_ids, e_ids, total = P.align(knobs["block_m"])
-            out = torch.zeros((M, shape.K), dtype=torch.bfloat16, device=dev)
-            byts.append(P.algorithmic_bytes())
-            flops.append(P.algorithmic_flops())
+    class Bench:
+        """Weights of one shape (rotated copies) and the measurement of one batch size on them."""
 
-            def call(P=P, W=W, s_ids=s_ids, e_ids=e_ids, total=total, out=out):
-                torch.ops.alpha_moe.fused_moe_w8a8_up_down(
-                    P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids, total, P.topk_weights, out,
-                    shape.top_k, knobs["block_m"], knobs["block_n"], knobs["warp_n"], knobs["stages"],
-                    shape.scaling_factor)
-            calls.append(call)
-        return calls, statistics.mean(byts), statistics.mean(flops), knobs, src
+        def __init__(self, name, cfg_path=None):
+            self.shape = SHAPES[name]
+            s = self.shape
+            self.cfg_path = cfg_path or os.path.join(ROOT, "alpha-moe_amd", "configs", f"moe_jit_{s.E}_{s.N}_{s.K}.json")
+            self.W0 = make_weights(s, device=dev, seed=0)
+            self.replicas = [self.W0]
+            for _ in range(max(1, args.replicas) - 1):
+                W0 = self.W0
+                self.replicas.append(Weights(s, W0.w1.clone(), W0.w1_scale.clone(), W0.w2.clone(), W0.w2_scale.clone()))
 
-    def measure(M, steps, warmup):
-        calls, B, F, knobs, src = prepare(M)
-        for i in range(warmup):
-            calls[i % len(calls)]()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(steps):
-            calls[i % len(calls)]()
-        torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-        # per-launch device time: HIP events on the launch stream (torch's current stream) around every call
-        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-        for i in range(steps):
-            evs[i][0].record()
-            calls[i % len(calls)]()
-            evs[i][1].record()
-        torch.cuda.synchronize()
-        dev_ms = [a.elapsed_time(b) for a, b in evs]
-        return {"M": M, "ms_per_step": wall_ms, "launch_us_mean": statistics.mean(dev_ms) * 1e3,
-                "launch_us_median": statistics.median(dev_ms) * 1e3, "launch_us_min": min(dev_ms) * 1e3,
-                "bytes": B, "flops": F, "knobs": knobs, "knobs_from": src}
+        def knobs_for(self, M):
+            if os.path.exists(self.cfg_path):
+                return dict(get_best_config(self.cfg_path, M)), os.path.relpath(self.cfg_path, ROOT)
+            return dict(DEFAULT_KNOBS), "built-in"
+
+        def prepare(self, M):
+            """Problems (routing + activations) for M tokens, one per routing seed, each bound to one weight replica."""
+            s = self.shape
+            knobs, src = self.knobs_for(M)
+            n_prob = n_routings if M <= 1024 else 3
+            calls, byts, flops = [], [], []
+            for i in range(n_prob):
+                W = self.replicas[i % len(self.replicas)]
+                P = make_problem(W, M, seed=i)
+                s_ids, e_ids, total = P.align(knobs["block_m"])
+                out = torch.zeros((M, s.K), dtype=torch.bfloat16, device=dev)
+                byts.append(P.algorithmic_bytes())
+                flops.append(P.algorithmic_flops())
+
+                def call(P=P, W=W, s_ids=s_ids, e_ids=e_ids, total=total, out=out):
+                    torch.ops.alpha_moe.fused_moe_w8a8_up_down(
+                        P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids, total, P.topk_weights, out,
+                        s.top_k, knobs["block_m"], knobs["block_n"], knobs["warp_n"], knobs["stages"], s.scaling_factor)
+                calls.append(call)
+            return calls, statistics.mean(byts), statistics.mean(flops), knobs, src
+
+        def measure(self, M, steps, warmup):
+            calls, B, F, knobs, src = self.prepare(M)
+            for i in range(warmup):
+                calls[i % len(calls)]()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(steps):
+                calls[i % len(calls)]()
+            torch.cuda.synchronize()
+            wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+            # per-launch device time: HIP events on the launch stream (torch's current stream) around every call
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+            for i in range(steps):
+                evs[i][0].record()
+                calls[i % len(calls)]()
+                evs[i][1].record()
+            torch.cuda.synchronize()
+            dev_ms = [a.elapsed_time(b) for a, b in evs]
+            return {"M": M, "ms_per_step": wall_ms, "launch_us_mean": statistics.mean(dev_ms) * 1e3,
+                    "launch_us_median": statistics.median(dev_ms) * 1e3, "launch_us_min": min(dev_ms) * 1e3,
+                    "bytes": B, "flops": F, "knobs": knobs, "knobs_from": src}
+
+    def summarise(r):
+        t_us = r["launch_us_mean"]
+        return {"us_per_layer": round(r["ms_per_step"] * 1e3, 2), "launch_us_mean": round(t_us, 2),
+                "launch_us_median": round(r["launch_us_median"], 2),
+                "algorithmic_MB": round(r["bytes"] / 1e6, 1), "GB_per_s": round(r["bytes"] / t_us / 1e3, 1),
+                "hbm_frac": round(r["bytes"] / t_us / 1e3 / HBM_PEAK_GBS, 4),
+                "TFLOP_per_s": round(r["flops"] / t_us / 1e6, 2),
+                "mfma_frac": round(r["flops"] / t_us / 1e6 / FP8_PEAK_TFLOPS, 5), "knobs": r["knobs"]}
+
+    def steps_for(M):
+        return max(10, min(args.steps, args.steps * 64 // max(M, 64) * 2))
 
     if args.calibrate_copy:
         src = torch.ones(1 << 28, dtype=torch.int32, device=dev)   # 1 GiB read + 1 GiB written per copy
@@ -130,21 +156,33 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    head = measure(args.M, args.steps, args.warmup)
-    others = args.also_M if args.also_M is not None else [m for m in (1, 4, 16, 64) if m != args.M]
-    per_M = {}
-    for m in [args.M] + list(others):
-        r = head if m == args.M else measure(m, max(20, args.steps // 2), args.warmup)
-        t_us = r["launch_us_mean"]
-        per_M[str(m)] = {
-            "us_per_layer": round(r["ms_per_step"] * 1e3, 2), "launch_us_mean": round(t_us, 2),
-            "launch_us_median": round(r["launch_us_median"], 2),
-            "algorithmic_MB": round(r["bytes"] / 1e6, 1), "GB_per_s": round(r["bytes"] / t_us / 1e3, 1),
-            "hbm_frac": round(r["bytes"] / t_us / 1e3 / HBM_PEAK_GBS, 4),
-            "TFLOP_per_s": round(r["flops"] / t_us / 1e6, 2),
-            "mfma_frac": round(r["flops"] / t_us / 1e6 / FP8_PEAK_TFLOPS, 5), "knobs": r["knobs"]}
+    bench = Bench(args.shape, args.config)
+    shape = bench.shape
+    head = bench.measure(args.M, args.steps, args.warmup)
+    default_others = DS_OTHER_M if args.shape == "ds" else OTHER_CONFIGS.get(args.shape, ())
+    others = args.also_M if args.also_M is not None else [m for m in default_others if m != args.M]
+    per_M = {str(args.M): summarise(head)}
+    for m in others:
+        per_M[str(m)] = summarise(bench.measure(m, steps_for(m), min(args.warmup, 5) if m > 64 else args.warmup))
+    per_M = dict(sorted(per_M.items(), key=lambda kv: int(kv[0])))
 
     achieved = head["bytes"] / head["launch_us_mean"] / 1e3   # GB/s
+    knobs_bm = head["knobs"]["block_m"]
+    if args.M >= 4096:   # prefill: the contraction is the bound (the weights stream once; from M ~ 8k the matrix time exceeds the HBM time)
+        tflops = head["flops"] / head["launch_us_mean"] / 1e6
+        roofline = {"bound": "mfma", "achieved": round(tflops, 1), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(tflops / FP8_PEAK_TFLOPS, 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.shape, args.M)),
+                    "kernel": "moe_tile_kernel" if knobs_bm > 32 else "moe_stream_kernel",
+                    "algorithmic_flops_per_launch": int(head["flops"]),
+                    "launch_us_mean": round(head["launch_us_mean"], 2)}
+    else:
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.shape, args.M)),
+                    "kernel": "moe_tile_kernel" if knobs_bm > 32 else "moe_stream_kernel",
+                    "algorithmic_bytes_per_launch": int(head["bytes"]),
+                    "launch_us_mean": round(head["launch_us_mean"], 2)}
     result = {
         "metric": "us_per_fused_moe_layer",
         "value": round(head["ms_per_step"] * 1e3, 2),
@@ -158,14 +196,10 @@ def main():
         "vs_baseline": None,
         "dtype": "fp8_e4m3",
         "data": "synthetic",
-        "config": {"workload": f"{shape.name}_decode_M{args.M}: E={shape.E} top_k={shape.top_k} K={shape.K} I={shape.I} "
-                               f"fp8 e4m3 128x128 block scales, {len(replicas)} weight copies x {n_routings} routings rotated",
+        "config": {"workload": f"{shape.name}_{'prefill' if args.M >= 512 else 'decode'}_M{args.M}: E={shape.E} top_k={shape.top_k} K={shape.K} I={shape.I} "
+                               f"fp8 e4m3 128x128 block scales, {len(bench.replicas)} weight copies x {n_routings} routings rotated",
                    "M": args.M, "knobs": head["knobs"], "knobs_from": head["knobs_from"]},
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.shape, args.M)),
-                     "kernel": "moe_stream_kernel", "algorithmic_bytes_per_launch": int(head["bytes"]),
-                     "launch_us_mean": round(head["launch_us_mean"], 2)},
+        "roofline": roofline,
         "per_M": per_M,
     }
 
@@ -173,6 +207,7 @@ def main():
         # the CPU port of the reference maths on the same bits, on this box's host cores (checker, not product)
         from oracle import moe_oracle as O
         torch.set_num_threads(os.cpu_count() or 1)
+        W0 = bench.W0
         Wc = Weights(shape, W0.w1.cpu(), W0.w1_scale.cpu(), W0.w2.cpu(), W0.w2_scale.cpu())
         P = make_problem(W0, args.M, seed=0)
         knobs = head["knobs"]
@@ -198,6 +233,19 @@ def main():
                                   "kind": "port", "sample": f"same call as the headline (M={args.M}, routing seed 0), "
                                                             f"median of {len(times)} runs of oracle/moe_oracle.py (torch fp32)"}
         result["parity"] = O.error_metrics(out, ref)
+        del Wc
+
+    if not args.no_other_configs and args.shape == "ds":
+        del bench
+        torch.cuda.empty_cache()
+        other = {}
+        for name, Ms in OTHER_CONFIGS.items():
+            b = Bench(name)
+            other[name] = {"shape": f"E={b.shape.E} top_k={b.shape.top_k} K={b.shape.K} I={b.shape.I}",
+                           "per_M": {str(m): summarise(b.measure(m, steps_for(m), min(args.warmup, 5))) for m in Ms}}
+            del b
+            torch.cuda.empty_cache()
+        result["other_configs"] = other
 
     print(json.dumps(result))
     return 0
