@@ -20,9 +20,14 @@
 //
 // There is no floating-point atomic anywhere: the result is bit-reproducible from run to run.
 //
-// Every wait is on items EARLIER in the queue, which are already held by running workgroups that never wait on
-// later ones, so the queue drains whatever the number of resident workgroups; each spin is bounded and sets
-// ctl->error instead of hanging.  The workspace starts zero-filled; its first kPrefixBytes hold the control block,
+// Every wait is on items EARLIER in the queue, and items never wait on later ones.  The first gridDim.x items belong to
+// the workgroups by index (no round trip to the counter, no storm of same-address atomics at the start), the rest
+// go to whoever asks the counter next.  The queue therefore drains as long as every workgroup of the grid becomes
+// resident without one of this launch's workgroups having to retire first: the host sizes the grid to what the
+// device holds at once (LDS granules included).  Another kernel occupying CUs only delays the items of the workgroups
+// it keeps out; two launches of THIS kernel that share a device at the same time could keep each other's workgroups
+// out for good, so launches on one device are serialised by the caller (one stream, or one workspace - which
+// concurrent launches may not share anyway).  Each spin is bounded and sets ctl->error instead of hanging.  The workspace starts zero-filled; its first kPrefixBytes hold the control block,
 // the arrival counters (reset by the last arrival) and epoch-stamped flags, so nothing has to be cleared between
 // launches; the rest (aq, sa, hpart, y) is only ever read after it was written in the same launch.
 //
@@ -192,8 +197,13 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     constexpr int TPK = NT + TM;            // ring tiles per wavefront per K block (token tiles first)
     constexpr int THREADS = WN * 64;
     static_assert(S >= 2 && 2 * (S - 1) < 64, "ring depth must fit the 6-bit vmcnt");
+    // The ring has one slot more than tiles in flight: the load issued at the top of a step then lands in the slot of the
+    // tile read TWO steps ago.  With S slots it would be the tile read one step ago, and a token tile's LDS read (nothing
+    // waits for it until the next matrix instruction) can still be queued when a fast load (the cached dummy line behind the
+    // end of an item) overwrites it: measured as one wavefront's 16 intermediate columns wrong in ~1 of 30 short UP items.
+    constexpr int R = S + 1;
 
-    // dynamic LDS: [WN rings of S tiles][n_ib * TM tiles of requantised activations (DOWN items)]
+    // dynamic LDS: [WN rings of S + 1 tiles][n_ib * TM tiles of requantised activations (DOWN items)]
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds_dyn[];
     __shared__ float s_sc[1024];                       // UP: gate scales [0,64), up scales [64,128); DOWN: w2 scales [blk][ib]
     __shared__ float s_xs[TM * 16][kItemKBlocks + 1];  // UP: activation scales [row][K block]; DOWN: sa [row][ib]
@@ -209,8 +219,8 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     const int n = lane & 15;
     const int q = lane >> 4;
     const int K = p.K, I = p.N >> 1;
-    uint8_t *ring = lds_dyn + wave * (S * 2048);
-    uint8_t *s_aq = lds_dyn + WN * (S * 2048);
+    uint8_t *ring = lds_dyn + wave * (R * 2048);
+    uint8_t *s_aq = lds_dyn + WN * (R * 2048);
 
     // operand read offsets inside a 16x128 tile (see the swizzle note at the top of the file)
     const int f_n = (n >> 1) & 7;
@@ -363,7 +373,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
 #pragma unroll
         for (int j = 0; j < S - 1; j++) {
             issue(j / TPK, j % TPK, slot_w);
-            slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
+            slot_w = slot_w + 1 == R ? 0 : slot_w + 1;
         }
         __syncthreads();   // s_xs is complete
         v8i bfrag[TM];
@@ -379,11 +389,11 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
 #pragma unroll
             for (int a = 0; a < TPK; a++) {
                 issue(kb + (a + S - 1) / TPK, (a + S - 1) % TPK, slot_w);
-                slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
+                slot_w = slot_w + 1 == R ? 0 : slot_w + 1;
                 __builtin_amdgcn_sched_barrier(0);
                 wait_vmcnt<2 * (S - 1)>();
                 const v8i frag = read_tile(ring + slot_r * 2048);
-                slot_r = slot_r + 1 == S ? 0 : slot_r + 1;
+                slot_r = slot_r + 1 == R ? 0 : slot_r + 1;
                 if (a < TM) {
                     bfrag[a < TM ? a : 0] = frag;
                 } else {
@@ -764,7 +774,7 @@ struct Variant {
 template <int TM, int WN, int S>
 Variant variant()
 {
-    return Variant{moe_stream_kernel<TM, WN, S>, WN * S * 2048, WN * 64, TM};
+    return Variant{moe_stream_kernel<TM, WN, S>, WN * (S + 1) * 2048, WN * 64, TM};
 }
 
 // `stages` sizes the LDS ring: 16 KiB per workgroup per stage, i.e. S = 8 * stages / WN tiles of 2 KiB per
@@ -822,6 +832,18 @@ hipError_t resident_slots(const Variant &v, int lds_bytes, int *slots)
     err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void *>(v.fn), v.threads,
                                                        lds_bytes);
     if (err != hipSuccess) return err;
+    // The runtime's answer divides the CU's LDS by the byte count; the hardware hands LDS out in granules (1280 bytes
+    // on gfx950), so three workgroups of 54 272 bytes each do NOT fit the 160 KiB although 3 * 54 272 < 163 840.  A grid
+    // one workgroup per CU too large is fatal here: the workgroups that are not resident own their first items (see
+    // the kernel's item loop) and the resident ones end up waiting for them.  Round up to both granules in use on
+    // CDNA parts and take the smaller count.
+    hipFuncAttributes attr;
+    err = hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(v.fn));
+    if (err != hipSuccess) return err;
+    const size_t need = attr.sharedSizeBytes + (size_t)lds_bytes;
+    const size_t g1 = (need + 1279) / 1280 * 1280, g2 = (need + 2047) / 2048 * 2048;
+    const int occ_lds = (int)(((size_t)160 << 10) / (g1 > g2 ? g1 : g2));
+    if (occ > occ_lds) occ = occ_lds;
     if (occ < 1) occ = 1;
     *slots = cus * occ;
     cache.push_back(Entry{v.fn, dev, lds_bytes, *slots});

@@ -149,3 +149,95 @@ def test_deepseek_shard_prefill_full_size_properties(ds_weights):
     assert torch.equal(out, run_op(P, 128, 64, 4, 3, via="c_abi"))
     print("case ds M=8192 knobs (64, 64, 4, 3)", flush=True)
     assert torch.equal(out, run_op(P, 64, 64, 4, 3, via="c_abi"))
+
+
+def _sampled_tokens_match_oracle(P, out, what, n=48, seed=11):
+    """A token's result depends on nothing but its own row, routing and the weights: recompute a sample on the CPU."""
+    from alpha_moe_python.workloads import Problem
+    gen = torch.Generator().manual_seed(seed)
+    idx = torch.randperm(P.M, generator=gen)[:n].sort().values.to(DEV)
+    sub = Problem(P.weights, n, P.x[idx].contiguous(), P.x_scale[idx].contiguous(), P.topk_ids[idx].contiguous(),
+                  P.topk_weights[idx].contiguous())
+    return assert_parity(out[idx], oracle_out(sub), what)
+
+
+@pytest.fixture(scope="module")
+def qn_weights():
+    return make_weights(SHAPES["qn"], device=DEV, seed=0)
+
+
+@pytest.mark.parametrize("M,knobs", [(1, (16, 32, 8, 5)), (32, (16, 32, 8, 5)), (256, (16, 64, 4, 3)), (256, (64, 64, 4, 3))])
+def test_qwen3_next_shard_against_oracle(qn_weights, M, knobs):
+    """Many small experts: E=512, top_k=10, K=2048, I=256, no shared expert (most experts idle at small M)."""
+    P = make_problem(qn_weights, M, seed=0)
+    print(f"case qn M={M} knobs {knobs}", flush=True)
+    m = assert_parity(run_op(P, *knobs, via="c_abi"), oracle_out(P), f"qn M={M} knobs {knobs}")
+    print("metrics", m, flush=True)
+
+
+def test_qwen3_next_shard_prefill_full_size(qn_weights):
+    P = make_problem(qn_weights, 4096, seed=1)
+    print("case qn M=4096 knobs (64, 32, 8, 2)", flush=True)
+    out = run_op(P, 64, 32, 8, 2, via="c_abi")
+    print("metrics", _sampled_tokens_match_oracle(P, out, "qn M=4096 sampled tokens"), flush=True)
+    print("case qn M=4096 knobs (128, 64, 4, 3)", flush=True)
+    assert torch.equal(out, run_op(P, 128, 64, 4, 3, via="c_abi"))
+
+
+@pytest.fixture(scope="module")
+def q3_weights():
+    return make_weights(SHAPES["q3"], device=DEV, seed=0)
+
+
+@pytest.mark.parametrize("M,knobs", [(64, (16, 32, 8, 5)), (64, (32, 64, 4, 3)), (200, (64, 64, 4, 3)), (200, (128, 64, 4, 2))])
+def test_qwen3_30b_zipf_shard_against_oracle(q3_weights, M, knobs):
+    """Load imbalance: E=128, top_k=8, K=2048, I=768 (six 128-column slices), Zipf(1.2) expert popularity.  Row blocks
+    of 128 rows do not fit the tile kernel's LDS budget with six slices and take the fallback kernel."""
+    P = make_problem(q3_weights, M, seed=0)
+    print(f"case q3 M={M} knobs {knobs}", flush=True)
+    m = assert_parity(run_op(P, *knobs, via="c_abi"), oracle_out(P), f"q3 M={M} knobs {knobs}")
+    print("metrics", m, flush=True)
+
+
+def test_qwen3_30b_zipf_shard_prefill_full_size(q3_weights):
+    P = make_problem(q3_weights, 8192, seed=1)
+    print("case q3 M=8192 knobs (64, 32, 8, 3)", flush=True)
+    out = run_op(P, 64, 32, 8, 3, via="c_abi")
+    print("metrics", _sampled_tokens_match_oracle(P, out, "q3 M=8192 sampled tokens"), flush=True)
+    print("case q3 M=8192 second launch", flush=True)
+    assert torch.equal(out, run_op(P, 64, 32, 8, 3, via="c_abi"))
+
+
+def test_short_up_items_repeat_launches():
+    """Many row blocks, short K: the UP items are a few K blocks long, so item starts, ends (loads pointed past the end
+    of an item) and LDS-ring reuse dominate.  Ten launches must all agree with the oracle and with each other."""
+    from alpha_moe_python.workloads import Shape
+    shape = Shape("short", E=512, top_k=10, K=1024, I=256, shared_expert=False, routing="softmax_renorm",
+                  scaling_factor=1.0)
+    W = make_weights(shape, device=DEV, seed=0)
+    P = make_problem(W, 32, seed=0)
+    ref = oracle_out(P)
+    for knobs in ((16, 32, 8, 5), (16, 32, 8, 2), (16, 64, 4, 1), (16, 64, 4, 2)):
+        print(f"case short M=32 knobs {knobs}", flush=True)
+        first = run_op(P, *knobs, via="c_abi")
+        assert_parity(first, ref, f"short M=32 knobs {knobs}")
+        for rep in range(9):
+            assert torch.equal(first, run_op(P, *knobs, via="c_abi")), (knobs, rep)
+
+
+@pytest.mark.parametrize("knobs", [(8, 64, 4, 2), (16, 64, 4, 5), (16, 32, 8, 4), (32, 64, 4, 3), (32, 32, 8, 5)])
+def test_grid_fits_the_device(ds_weights, knobs):
+    """The workgroups of a launch wait for each other, so the grid must not exceed what the device holds at once -
+    also for ring sizes where the LDS allocation granule decides how many workgroups fit a CU.  A grid that is too
+    large shows as a launch that takes seconds (bounded waits running out) and as wrong results."""
+    import time
+    P = make_problem(ds_weights, 64, seed=0)
+    print(f"case ds M=64 knobs {knobs}", flush=True)
+    run_op(P, *knobs, via="c_abi")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = run_op(P, *knobs, via="c_abi")
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert dt < 0.5, f"launch took {dt:.2f} s"
+    assert_parity(out, oracle_out(P), f"ds M=64 knobs {knobs}")
