@@ -106,7 +106,10 @@ struct StreamCtl {
     int epoch;       // completed launches on this workspace (any kernel family)
     int error;       // sticky: a bounded wait ran out
     int fin_done;    // tile kernels: reduce-kernel workgroups that have left
-    int pad0[27];
+    int tile_done;   // tile kernel: workgroups that have left
+    int pad0[2];
+    int tile_head[8];   // tile kernel: next work item of each of the eight queues
+    int pad1a[16];
     // a 128-byte line of its own: idle workgroups poll it while the others still fetch items through `head`
     int down_done;   // streaming kernel: finished DOWN items of this launch
     int pad1[31];

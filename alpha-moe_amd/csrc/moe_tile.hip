@@ -1,38 +1,40 @@
-// Fused W8A8 MoE, "tile" kernel for large batches: one workgroup of 8 wavefronts (two per SIMD) per row block of
-// block_m sorted rows.
+// Fused W8A8 MoE, "tile" kernel for large batches: persistent workgroups of 8 wavefronts (two per SIMD, one workgroup
+// per compute unit) that take work items from eight queues.  A row block of block_m sorted rows is I/128 UP items (one
+// 128-column slice of the intermediate each) and a few DOWN items (a slab of output columns each).
 //
-// Up/gate projection.  The workgroup walks the I/128 slices of the intermediate one after the other.  For a slice it
-// contracts its 256 interleaved w1 rows against the block's tokens over all of K, one 128-byte K block per step.
-// Every operand reaches the matrix cores through LDS, filled by direct-to-LDS loads that cover whole 128-byte lines:
-// measured on MI355X, a compute unit takes ~38 GB/s from L2 when a load instruction touches 16 rows x 64 bytes (the
-// matrix-operand register layout) and ~100 GB/s when it touches 8 rows x 128 bytes, and at full matrix rate a
-// 128-token block needs ~110 GB/s.  Wavefront (w, g) multiplies weight rows 64 w .. 64 w + 63 (4 operand tiles) with
-// token half g; the two wavefronts of a pair w share a 3-stage ring of weight tiles and each loads half of it; the
-// token tiles (16 tokens x 128 bytes, gathered through the routing) and their scales go through a 3-stage ring shared
-// by everybody, one tile per wavefront, with one workgroup barrier per step.  A wavefront issues 4 x TH matrix
+// UP item.  The workgroup contracts the slice's 256 interleaved w1 rows against the block's tokens over all of K, one
+// 128-byte K block per step.  Every operand reaches the matrix cores through LDS, filled by direct-to-LDS loads that
+// cover whole 128-byte lines: measured on MI355X, a compute unit takes ~38 GB/s from L2 when a load instruction touches
+// 16 rows x 64 bytes (the matrix-operand register layout) and ~100 GB/s when it touches 8 rows x 128 bytes, and at full
+// matrix rate a 128-token block needs ~110 GB/s.  Wavefront (w, g) multiplies weight rows 64 w .. 64 w + 63 (4 operand
+// tiles) with token half g; the two wavefronts of a pair w share a 3-stage ring of weight tiles and each loads half of
+// it; the token tiles (16 tokens x 128 bytes, gathered through the routing) and their scales go through a 3-stage ring
+// shared by everybody, one tile per wavefront, with one workgroup barrier per step.  A wavefront issues 4 x TH matrix
 // instructions per step; the 4 multiply-adds that scale a 16x16 product into the fp32 accumulators are placed right
 // behind the NEXT matrix instruction so that vector and matrix pipes overlap (75% of the FP8 peak for this loop in
 // isolation against 35% when the compiler orders it), and the step's loads are spread between them: a direct-to-LDS
 // load blocks the issuing wavefront for 30-60 ns, during which the SIMD's other wavefront computes.
+// SwiGLU and the FP8 requantisation of the 128-column group happen in registers (cross-wavefront amax through LDS);
+// the block_m x 128 FP8 tile goes to a scratch area of the workspace in operand-tile layout, its per-token scales
+// beside it, and the unit's flag is stamped with the launch epoch.
 //
-// What bounds it (measured, M = 8192 on the DeepSeek-V3 shard): a step takes ~1.5 us against 0.43 us of matrix time.
-// A compute unit keeps about 32 KiB of L2 misses in flight whatever the ring depth (two or three stages, one or four
-// wavefronts issuing: same rate), so its load rate is 32 KiB / latency: ~100 GB/s on L2 hits, ~40 GB/s on misses; the
-// first block of an expert misses on all 48 KiB of a step, and the blocks sharing its weights follow at its pace.
-//
-// SwiGLU and the FP8 requantisation of the 128-column group happen in registers (cross-wavefront amax through LDS).
-// LDS is full of rings at that point, so the block_m x 128 FP8 tile is parked in a scratch area of the workspace (it
-// stays in L2) in operand-tile layout and fetched back into LDS, where the token ring was, once all slices are done.
-//
-// Down projection.  64 output columns at a time (4 operand tiles of w2 rows through the pair's ring), all slices,
-// the wavefront's token half.  The w2 rows of a tile are picked so that a lane ends up with 16 adjacent output columns
-// of its token: each valid (token, slot) row is written ONCE, in bf16, as whole 128-byte lines, to y[slot]: top_k
-// result rows per token instead of the top_k * I/128 partial rows the reference's decomposition
+// DOWN item.  Waits for the flags of the block's slices, fetches their tiles and scales into LDS (where the token ring
+// was) and contracts them with w2: 64 output columns at a time (4 operand tiles of w2 rows through the pair's ring),
+// all slices, the wavefront's token half.  The w2 rows of a tile are picked so that a lane ends up with 16 adjacent
+// output columns of its token: each valid (token, slot) row is written ONCE, in bf16, as whole 128-byte lines, to
+// y[slot]: top_k result rows per token instead of the top_k * I/128 partial rows the reference's decomposition
 // (fused_moe_w8a8_up_down_acc.cu:676-679,1085-1091) adds into the output.  A second kernel sums a token's live rows
 // in fp32 and rounds into `out` once.  No atomics: at M = 8192 fp32 atomics alone cost 13 ms on MI355X.
 //
-// Workgroups are renumbered so that consecutive row blocks (the blocks of one expert) run on the same XCD and share
-// its L2: the hardware deals workgroup i to XCD i % 8.
+// What bounds it (measured on the DeepSeek-V3 shard): a compute unit keeps about 32 KiB of L2 misses in flight whatever
+// the ring depth (two or three stages, one or four wavefronts issuing: same rate), so alone it streams ~37 GB/s and a
+// step takes ~1.5 us against 0.43 us of matrix time; 256 of them together reach what HBM and the fabric deliver.
+// Everything therefore hinges on keeping all compute units busy and on the bytes they pull: items instead of whole row
+// blocks (one workgroup per block left 16 of 272 blocks at M = 1024 to a second round: 547 us, now 391 us), the
+// blocks of one expert next to each other on one XCD so that they share its L2, and non-temporal loads for the
+// weights of experts that have a single block.
+#include <stdlib.h>
+
 #include "moe_common.hpp"
 
 namespace alpha_moe {
@@ -48,24 +50,16 @@ constexpr int kMaxTailBytes = 48 << 10;           // token-tile ring / requantis
 struct TileParams {
     MoeParams p;
     StreamCtl *ctl;
+    int *flag;        // [row blocks][n_ib] == epoch once the unit's requantised tiles are in scratch
     int *live;        // [slots] == epoch once y[slot] is written this launch
     uint16_t *y;      // [slots][K] bf16
     uint8_t *aqs;     // [row blocks][n_ib][TM] requantised operand tiles of 2 KiB
+    float *sas;       // [row blocks][n_ib][TM * 16] their per-token scales
     int n_ib, nkb, n_mb_max;
+    int gps, n_cs;    // 64-column groups per DOWN item, DOWN items per row block
+    int lag;          // row blocks whose up/gate items precede the first down items of a queue
+    int w_nt;         // weights with non-temporal loads: 1 always, 0 never, -1 for experts with a single row block
 };
-
-#ifdef ALPHA_MOE_TRACE
-// Debug builds only: 100 MHz wall-clock stamps of wavefront 0 per up/gate step: loads landed, barrier passed, next
-// loads issued, step computed.
-// Stamps are kept in LDS during the kernel (a global store would join the vector-memory queue that the step
-// loop counts) and written out at the end.
-constexpr int kTraceSteps = 112;
-__device__ unsigned int g_tile_trace[1024][kTraceSteps][4];
-#define TILE_STAMP(step, i)                                                                       \
-    if (tid == 0 && (step) < kTraceSteps) s_trace[step][i] = (unsigned int)wall_clock64()
-#else
-#define TILE_STAMP(step, i)
-#endif
 
 typedef const void __attribute__((address_space(1))) * gptr_t;
 typedef void __attribute__((address_space(3))) * lptr_t;
@@ -74,6 +68,11 @@ typedef void __attribute__((address_space(3))) * lptr_t;
 __device__ __forceinline__ void dma16(const void *g, void *lds)
 {
     __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uintptr_t)lds, 16, 0, 0);
+}
+// the same, non-temporal: for weight streams that nobody else reads soon (see the streaming kernel's header for the rates)
+__device__ __forceinline__ void dma16_nt(const void *g, void *lds)
+{
+    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uintptr_t)lds, 16, 0, 2);
 }
 __device__ __forceinline__ void dma4(const void *g, void *lds)
 {
@@ -151,6 +150,36 @@ __device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *
     for (int k = 0; k < 4; k++) acc[k][TH - 1] += prev[k] * ((k & 1) ? p1 : p0);
 }
 
+// Agent-scope accesses for what crosses workgroups (and XCDs, whose L2s are not coherent with each other) inside the
+// launch: requantised tiles, their scales, the flags.
+__device__ __forceinline__ void stg32_agent(void *p, uint32_t v)
+{
+    asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+}
+__device__ __forceinline__ void dma16_agent(const void *g, void *lds)
+{
+    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uintptr_t)lds, 16, 0, 16);   // sc1
+}
+__device__ __forceinline__ int load_agent(const int *p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_agent(int *p, int v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Bounded wait of one thread for *addr >= target: ~4M polls a microsecond apart, then the sticky error flag.
+__device__ __noinline__ void tile_spin_until_ge(const int *addr, int target, StreamCtl *ctl)
+{
+    for (int it = 0; it < (1 << 22); it++) {
+        if (load_agent(addr) >= target) return;
+        if (it < 16) __builtin_amdgcn_s_sleep(4);
+        else __builtin_amdgcn_s_sleep(32);
+    }
+    store_agent(&ctl->error, 1);
+}
+
 // TH: 16-token tiles per wavefront; a row block has TM = 2 TH of them (block_m rounded up to 32 rows).
 // Wavefront v = (w = v % 4, g = v / 4): weight rows 64 w .. 64 w + 63 of the slice, token tiles g TH .. g TH + TH - 1.
 template <int TH>
@@ -162,8 +191,8 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
     constexpr int XOPS = 3;                   // one token tile (2 halves) + its 16 scales
     constexpr int OPS1 = AOPS + XOPS;
 
-    // [4 pairs][3 stages][4 tiles] weight rings | [3 stages][TM] token tiles; the requantised tiles [n_ib][TM]
-    // later take the place of the token tiles
+    // [4 pairs][3 stages][4 tiles] weight rings | UP items: [3 stages][TM] token tiles; DOWN items: the requantised
+    // tiles [n_ib][TM] in the same place
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds_dyn[];
     __shared__ __attribute__((aligned(1024))) uint8_t s_dummy[2048 + 64];
     __shared__ float s_xs[kStages][TM * 16];
@@ -172,20 +201,9 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
     __shared__ float s_sa[kTileMaxIb][TM * 16];
     __shared__ float s_w2s[kTileMaxW2s];
     __shared__ int s_tok[TM * 16];
-#ifdef ALPHA_MOE_TRACE
-    __shared__ unsigned int s_trace[kTraceSteps][4];
-#endif
+    __shared__ int s_item[2];
 
     const MoeParams &p = s.p;
-    // consecutive row blocks on one XCD: workgroup i runs on XCD i % 8
-    int n_live = (p.ntpp[0] + p.block_m - 1) / p.block_m;
-    n_live = n_live < s.n_mb_max ? n_live : s.n_mb_max;
-    const int per_xcd = (n_live + 7) >> 3;
-    const int mb = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-    if ((int)(blockIdx.x >> 3) >= per_xcd || mb >= n_live) return;
-    const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
-    if (e < 0 || e >= p.E) return;
-
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -198,6 +216,14 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
     uint8_t *a_ring = lds_dyn + w * (kStages * 8192);
     uint8_t *xbuf = lds_dyn + kARingBytes;
 
+    // Row blocks are dealt to eight queues in contiguous runs (the blocks of one expert are neighbours), and a
+    // workgroup serves the queue of its XCD first (the hardware deals workgroup i to XCD i % 8): the workgroups that
+    // stream the same expert's weights at the same time then share one L2.
+    int n_live = (__builtin_amdgcn_readfirstlane(p.ntpp[0]) + p.block_m - 1) / p.block_m;
+    n_live = n_live < s.n_mb_max ? n_live : s.n_mb_max;
+    const int per_q = (n_live + 7) >> 3;
+    const int per_up = n_ib, per_down = s.n_cs;
+
     // operand fragment of lane (n, q): chunks q and q+4 of row n; chunk c of row r sits at position c ^ ((r >> 1) & 7)
     const int f_n = (n >> 1) & 7;
     const int frag_lo = n * 128 + 16 * (q ^ f_n);
@@ -208,66 +234,64 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
 #pragma unroll
     for (int h = 0; h < 2; h++) ld_chunk[h] = 16 * ((lane & 7) ^ (((8 * h + ld_row) >> 1) & 7));
 
-    // ---- routing ---------------------------------------------------------------------------------------------
-    int slot[TH];
-    bool valid[TH];
-#pragma unroll
-    for (int t = 0; t < TH; t++) {
-        const int row = (g * TH + t) * 16 + n;
-        const int idx = mb * p.block_m + row;
-        int id = -1;
-        if (row < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
-        valid[t] = id >= 0 && id / p.top_k < p.M;
-        slot[t] = valid[t] ? id : 0;
-        if (w == 0 && q == 0 && valid[t]) s.live[slot[t]] = epoch;
-    }
-    if (tid < TM * 16) {
-        const int idx = mb * p.block_m + tid;
-        int id = -1;
-        if (tid < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
-        const int tk = id / p.top_k;
-        s_tok[tid] = (id >= 0 && tk < p.M) ? tk : 0;
-    }
-    for (int i = tid; i < (K >> 7) * n_ib; i += THREADS) s_w2s[i] = p.w2_scale[(size_t)e * (K >> 7) * n_ib + i];
-    __syncthreads();
+    v4f acc[4][TH];
 
-    // token-tile gather: wavefront v loads tile v (a dummy where the block has no such tile)
-    const bool x_real = wave < TM;
-    const uint8_t *gx[2];
-#pragma unroll
-    for (int h = 0; h < 2; h++) gx[h] = p.x + (size_t)s_tok[x_real ? wave * 16 + 8 * h + ld_row : 0] * K + ld_chunk[h];
-    const float *gxs = p.x_scale + (size_t)s_tok[x_real ? wave * 16 + (lane & 15) : 0] * nkb;
-    auto issue_x_op = [&](int kb, int stage, int part) {   // operation `part` of XOPS
-        const int kc = kb < nkb ? kb : nkb - 1;
-        if (part < 2) {
-            uint8_t *dst = x_real ? xbuf + stage * (TM * 2048) + wave * 2048 : s_dummy;
-            dma16(gx[part] + (size_t)kc * 128, dst + part * 1024);
-        } else {
-            float *sdst = x_real ? &s_xs[stage][wave * 16] : reinterpret_cast<float *>(s_dummy + 2048);
-            if (lane < 16) dma4(gxs + kc, sdst);
-        }
+    // ---- UP item: slice ib of row block mb -> requantised operand tiles + scales in scratch, then the unit's flag ----
+    // An expert with a single row block streams its weights with non-temporal loads (measured on the DeepSeek-V3 shard:
+    // -13 % at M = 512 where nearly every expert has one block, +8 % at M = 8192 if applied to experts whose blocks run
+    // side by side and share the lines in L2).
+    auto lone_block = [&](int mb, int e) {
+        if (s.w_nt >= 0) return s.w_nt != 0;
+        const bool left = mb > 0 && __builtin_amdgcn_readfirstlane(p.expert_ids[mb - 1]) == e;
+        const bool right = mb + 1 < n_live && __builtin_amdgcn_readfirstlane(p.expert_ids[mb + 1]) == e;
+        return !left && !right;
     };
 
-    v4f acc[4][TH];
-    for (int ib = 0; ib < n_ib; ib++) {
+    auto up_item = [&](int mb, int ib) {
+        const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
+        if (e < 0 || e >= p.E) return;
+        const bool nt = lone_block(mb, e);
+        if (tid < TM * 16) {
+            const int idx = mb * p.block_m + tid;
+            int id = -1;
+            if (tid < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
+            const int tk = id / p.top_k;
+            s_tok[tid] = (id >= 0 && tk < p.M) ? tk : 0;
+        }
         // this slice's gate (row 2*ib) and up (row 2*ib+1) scale rows
         {
             const float *ws_rows = p.w_scale + ((size_t)e * (p.N >> 7) + 2 * ib) * nkb;
             for (int i = tid; i < 2 * nkb; i += THREADS) s_ws[i >= nkb][i >= nkb ? i - nkb : i] = ws_rows[i];
         }
+        __syncthreads();
+
+        // token-tile gather: wavefront v loads tile v (a dummy where the block has no such tile)
+        const bool x_real = wave < TM;
+        const uint8_t *gx[2];
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+            gx[h] = p.x + (size_t)s_tok[x_real ? wave * 16 + 8 * h + ld_row : 0] * K + ld_chunk[h];
+        const float *gxs = p.x_scale + (size_t)s_tok[x_real ? wave * 16 + (lane & 15) : 0] * nkb;
         // Weight rows of the pair: tile a = (32-row group a / 2, gate | up a % 2); matrix row r of the tile is slab row
         // group * 32 + (r / 8) * 16 + r % 8 (+ 8 for up), so load h of a tile covers slab rows ... + 16 h + lane / 8.
         // Wavefront (w, g) loads tiles 2g and 2g + 1 of pair w.
         const uint8_t *wbase = p.w + ((size_t)e * p.N + ib * 256 + w * 64 + g * 32 + ld_row) * K;
-        // operation i of a step's OPS1: weight tile half (i < AOPS) or a token-tile operation
+        // operation i of a step's OPS1: weight tile half (i < AOPS), token tile half, token scales
         auto issue_op = [&](int kb, int stage, int i) {
+            const int kc = kb < nkb ? kb : nkb - 1;
             if (i < AOPS) {
-                const int kc = kb < nkb ? kb : nkb - 1;
                 const int up = i >> 1, h = i & 1;
-                dma16(wbase + (size_t)(h * 16 + 8 * up) * K + (size_t)kc * 128 + ld_chunk[h],
-                      a_ring + stage * 8192 + (2 * g + up) * 2048 + h * 1024);
+                const uint8_t *src = wbase + (size_t)(h * 16 + 8 * up) * K + (size_t)kc * 128 + ld_chunk[h];
+                uint8_t *dst = a_ring + stage * 8192 + (2 * g + up) * 2048 + h * 1024;
+                if (nt) dma16_nt(src, dst);
+                else dma16(src, dst);
+            } else if (i < AOPS + 2) {
+                const int part = i - AOPS;
+                uint8_t *dst = x_real ? xbuf + stage * (TM * 2048) + wave * 2048 : s_dummy;
+                dma16(gx[part] + (size_t)kc * 128, dst + part * 1024);
             } else {
-                issue_x_op(kb, stage, i - AOPS);
+                float *sdst = x_real ? &s_xs[stage][wave * 16] : reinterpret_cast<float *>(s_dummy + 2048);
+                if (lane < 16) dma4(gxs + kc, sdst);
             }
         };
         auto issue_all = [&](int kb, int stage) {
@@ -282,7 +306,6 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         // Per wavefront the loads of step kb are issued two steps ahead.  Step kb: wait for the own loads of kb (those of
         // kb + 1 stay in flight), meet the others (their tiles of kb have landed, and everybody is done reading
         // stage (kb + 2) % 3), then compute while refilling that stage.
-        __syncthreads();   // s_ws written; everybody is done with the previous slice
         issue_all(0, 0);
         issue_all(1, 1);
         for (int kb0 = 0; kb0 < nkb; kb0 += kStages) {
@@ -291,21 +314,17 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
                 const int kb = kb0 + h;
                 if (kb < nkb) {
                     wait_vmcnt<OPS1>();
-                    TILE_STAMP(ib * nkb + kb, 0);
                     lds_barrier();
-                    TILE_STAMP(ib * nkb + kb, 1);
-                    TILE_STAMP(ib * nkb + kb, 2);
                     mma_step<TH, OPS1>(a_ring + h * 8192, xbuf + h * (TM * 2048) + g * (TH * 2048),
                                        &s_xs[h][g * (TH * 16) + n], s_ws[0][kb], s_ws[1][kb], acc, frag_lo, frag_hi,
                                        [&](int i) { issue_op(kb + 2, (h + 2) % kStages, i); });
                     __builtin_amdgcn_sched_barrier(0);
-                    TILE_STAMP(ib * nkb + kb, 3);
                 }
             }
         }
         wait_vmcnt<0>();
 
-        // ---- SwiGLU, per-token amax over the slice's 128 columns, FP8 requant into operand tiles (scratch) ---------
+        // SwiGLU, per-token amax over the slice's 128 columns, FP8 requant into operand tiles
 #pragma unroll
         for (int t = 0; t < TH; t++) {
             float m = 0.f;
@@ -322,6 +341,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
             if (q == 0) s_amax[w][(g * TH + t) * 16 + n] = m;
         }
         __syncthreads();
+        const int unit = mb * n_ib + ib;
 #pragma unroll
         for (int t = 0; t < TH; t++) {
             const int tg = g * TH + t;
@@ -329,113 +349,214 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
 #pragma unroll
             for (int wv = 0; wv < 4; wv++) m = fmaxf(m, s_amax[wv][tg * 16 + n]);
             const float s_a = m / kFp8Max;
-            uint8_t *tile = s.aqs + ((size_t)(mb * n_ib + ib) * TM + tg) * 2048;
+            uint8_t *tile = s.aqs + ((size_t)unit * TM + tg) * 2048;
 #pragma unroll
             for (int pr = 0; pr < 2; pr++) {
                 const uint32_t packed =
                     pack_fp8x4(clamp_fp8(acc[2 * pr][t][0] / s_a), clamp_fp8(acc[2 * pr][t][1] / s_a),
                                clamp_fp8(acc[2 * pr][t][2] / s_a), clamp_fp8(acc[2 * pr][t][3] / s_a));
                 // columns w*32 + pr*16 + 4q .. +3 of token n: chunk w*2 + pr of the row, bytes 4q .. 4q+3 in it
-                *reinterpret_cast<uint32_t *>(tile + n * 128 + 16 * ((w * 2 + pr) ^ f_n) + 4 * q) = packed;
+                stg32_agent(tile + n * 128 + 16 * ((w * 2 + pr) ^ f_n) + 4 * q, packed);
             }
-            if (w == 0 && q == 0) s_sa[ib][tg * 16 + n] = s_a;
+            if (w == 0 && q == 0) stg32_agent(&s.sas[(size_t)unit * (TM * 16) + tg * 16 + n], __builtin_bit_cast(uint32_t, s_a));
         }
-    }
-    // the requantised tiles come back from scratch (L2) into LDS where the token ring was
-    __syncthreads();   // also waits for this wavefront's scratch stores
-#ifdef ALPHA_MOE_TRACE
-    if (blockIdx.x < 1024)
-        for (int i = tid; i < kTraceSteps * 4; i += THREADS) (&g_tile_trace[blockIdx.x][0][0])[i] = (&s_trace[0][0])[i];
-#endif
-    uint8_t *aq = xbuf;
-    for (int i = wave; i < n_ib * TM; i += 8) {
-        const uint8_t *src = s.aqs + ((size_t)mb * n_ib * TM + i) * 2048 + lane * 16;
-        dma16(src, aq + i * 2048);
-        dma16(src + 1024, aq + i * 2048 + 1024);
-    }
-    wait_vmcnt<0>();
-    __syncthreads();
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (tid == 0) store_agent(&s.flag[unit], epoch);
+    };
 
-    // ---- down projection: 64 output columns per step group, all slices ---------------------------------------------
-    // Pair w takes column groups w, w + 4, ...; its two wavefronts split the tokens as before and each loads two of the
-    // four w2 tiles of a step.  Matrix row r of tile k is output column c0 + 16 (r / 4) + 4 k + r % 4, so lane (n, q)
-    // collects columns c0 + 16 q .. c0 + 16 q + 15 of token n over the four tiles.  Load h of a tile: rows 8h + lane / 8.
-    float tw[TH];
+    // ---- DOWN item: column groups [cs * gps, (cs + 1) * gps) of row block mb, all slices ------------------------------
+    // 64 output columns per step group.  Pair w takes the slab's groups w, w + 4, ...; its two wavefronts split the
+    // tokens as before and each loads two of the four w2 tiles of a step.  Matrix row r of tile k is output column
+    // c0 + 16 (r / 4) + 4 k + r % 4, so lane (n, q) collects columns c0 + 16 q .. c0 + 16 q + 15 of token n over the
+    // four tiles.  Load h of a tile: rows 8h + lane / 8.
+    auto down_item = [&](int mb, int cs) {
+        const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
+        if (e < 0 || e >= p.E) return;
+        const bool nt = lone_block(mb, e);
+        int slot[TH];
+        bool valid[TH];
+        float tw[TH];
 #pragma unroll
-    for (int t = 0; t < TH; t++) tw[t] = valid[t] ? p.topk_w[slot[t]] * p.scaling : 0.f;
-    const int n_groups = K >> 6;
-    const int my_groups = (n_groups - w + 3) >> 2;            // column groups w, w + 4, ...
-    const int n_steps = ((n_groups + 3) >> 2) * n_ib;         // (group, slice) steps of the longest pair, slice-minor
-    const uint8_t *w2base = p.w2 + ((size_t)e * K + 16 * (lane >> 5) + (ld_row & 3)) * I;
-    int lg = 0, lib = 0;   // (group index, slice) of the next step to load
-    auto issue2_op = [&](int stage, int i) {   // operation i of AOPS of the step (lg, lib)
-        const int gc = lg < my_groups ? lg : my_groups - 1;
-        const int c0 = (w + 4 * gc) << 6;
-        const int k = 2 * g + (i >> 1), h = i & 1;
-        dma16(w2base + (size_t)(c0 + 32 * h + 4 * k) * I + lib * 128 + ld_chunk[h],
-              a_ring + stage * 8192 + k * 2048 + h * 1024);
-    };
-    auto advance2 = [&]() {
-        lib++;
-        if (lib == n_ib) {
-            lib = 0;
-            lg++;
+        for (int t = 0; t < TH; t++) {
+            const int row = (g * TH + t) * 16 + n;
+            const int idx = mb * p.block_m + row;
+            int id = -1;
+            if (row < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
+            valid[t] = id >= 0 && id / p.top_k < p.M;
+            slot[t] = valid[t] ? id : 0;
+            tw[t] = valid[t] ? p.topk_w[slot[t]] * p.scaling : 0.f;
+            if (cs == 0 && w == 0 && q == 0 && valid[t]) s.live[slot[t]] = epoch;
         }
-    };
-    auto issue2 = [&](int stage) {
+        for (int i = tid; i < (K >> 7) * n_ib; i += THREADS) s_w2s[i] = p.w2_scale[(size_t)e * (K >> 7) * n_ib + i];
+
+        const int n_groups = K >> 6;
+        const int g0 = cs * s.gps;
+        const int g1 = g0 + s.gps < n_groups ? g0 + s.gps : n_groups;
+        const int span = g1 - g0;
+        int my_groups = (span - w + 3) >> 2;                      // the slab's groups w, w + 4, ... (none: 0)
+        my_groups = my_groups > 0 ? my_groups : 0;
+        const int n_steps = ((span + 3) >> 2) * n_ib;             // (group, slice) steps of the longest pair, slice-minor
+        const uint8_t *w2base = p.w2 + ((size_t)e * K + 16 * (lane >> 5) + (ld_row & 3)) * I;
+        int lg = 0, lib = 0;   // (group index, slice) of the next step to load
+        auto group_of = [&](int i) {   // i-th group of this pair, clamped into the slab for loads past its end
+            int grp = g0 + w + 4 * (i < my_groups ? i : my_groups - 1);
+            grp = grp < g0 ? g0 : grp;
+            return grp < g1 ? grp : g1 - 1;
+        };
+        auto issue2_op = [&](int stage, int i) {   // operation i of AOPS of the step (lg, lib)
+            const int c0 = group_of(lg) << 6;
+            const int k = 2 * g + (i >> 1), h = i & 1;
+            const uint8_t *src = w2base + (size_t)(c0 + 32 * h + 4 * k) * I + lib * 128 + ld_chunk[h];
+            uint8_t *dst = a_ring + stage * 8192 + k * 2048 + h * 1024;
+            if (nt) dma16_nt(src, dst);
+            else dma16(src, dst);
+        };
+        auto advance2 = [&]() {
+            lib++;
+            if (lib == n_ib) {
+                lib = 0;
+                lg++;
+            }
+        };
+        auto issue2 = [&](int stage) {
 #pragma unroll
-        for (int i = 0; i < AOPS; i++) issue2_op(stage, i);
-        advance2();
-    };
+            for (int i = 0; i < AOPS; i++) issue2_op(stage, i);
+            advance2();
+        };
+        // the weights do not depend on the up/gate phase: first two steps go out before the wait
+        issue2(0);
+        issue2(1);
+        if (tid == 0)
+            for (int ib = 0; ib < n_ib; ib++) tile_spin_until_ge(&s.flag[mb * n_ib + ib], epoch, s.ctl);
+        __syncthreads();
+        // the requantised tiles and their scales come from scratch into LDS
+        uint8_t *aq = xbuf;
+        for (int i = wave; i < n_ib * TM; i += 8) {
+            const uint8_t *src = s.aqs + ((size_t)mb * n_ib * TM + i) * 2048 + lane * 16;
+            dma16_agent(src, aq + i * 2048);
+            dma16_agent(src + 1024, aq + i * 2048 + 1024);
+        }
+        for (int i = tid; i < n_ib * TM * 16; i += THREADS) {
+            const int bits = load_agent(reinterpret_cast<const int *>(&s.sas[(size_t)mb * n_ib * (TM * 16) + i]));
+            s_sa[i / (TM * 16)][i % (TM * 16)] = __builtin_bit_cast(float, bits);
+        }
+        wait_vmcnt<0>();
+        __syncthreads();
+
 #pragma unroll
-    for (int a = 0; a < 4; a++)
+        for (int a = 0; a < 4; a++)
 #pragma unroll
-        for (int t = 0; t < TH; t++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
-    int cg = 0, cib = 0;
-    issue2(0);
-    issue2(1);
-    for (int s0 = 0; s0 < n_steps; s0 += kStages) {
+            for (int t = 0; t < TH; t++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+        int cg = 0, cib = 0;
+        // the ring's first two steps were issued above and have landed (wait_vmcnt<0>): from here on one younger step
+        // stays in flight
+        for (int s0 = 0; s0 < n_steps; s0 += kStages) {
 #pragma unroll
-        for (int h = 0; h < kStages; h++) {
-            if (s0 + h < n_steps) {
-                // one younger step of AOPS loads stays in flight; result stores only make this stricter
-                wait_vmcnt<AOPS>();
-                lds_barrier();
-                const int gcl = cg < my_groups ? cg : my_groups - 1;
-                const int c0 = (w + 4 * gcl) << 6;
-                const float ws2 = s_w2s[(c0 >> 7) * n_ib + cib];
-                mma_step<TH, AOPS>(a_ring + h * 8192, aq + cib * (TM * 2048) + g * (TH * 2048),
-                                   &s_sa[cib][g * (TH * 16) + n], ws2, ws2, acc, frag_lo, frag_hi,
-                                   [&](int i) { issue2_op((h + 2) % kStages, i); });
-                advance2();
-                __builtin_amdgcn_sched_barrier(0);
-                cib++;
-                if (cib == n_ib) {
+            for (int h = 0; h < kStages; h++) {
+                if (s0 + h < n_steps) {
+                    // one younger step of AOPS loads stays in flight; result stores only make this stricter
+                    wait_vmcnt<AOPS>();
+                    lds_barrier();
+                    const int c0 = group_of(cg) << 6;
+                    const float ws2 = s_w2s[(c0 >> 7) * n_ib + cib];
+                    mma_step<TH, AOPS>(a_ring + h * 8192, aq + cib * (TM * 2048) + g * (TH * 2048),
+                                       &s_sa[cib][g * (TH * 16) + n], ws2, ws2, acc, frag_lo, frag_hi,
+                                       [&](int i) { issue2_op((h + 2) % kStages, i); });
+                    advance2();
+                    __builtin_amdgcn_sched_barrier(0);
+                    cib++;
+                    if (cib == n_ib) {
 #pragma unroll
-                    for (int t = 0; t < TH; t++) {
-                        if (valid[t] && cg < my_groups) {
-                            uint16_t *yp = s.y + (size_t)slot[t] * K + c0 + 16 * q;
+                        for (int t = 0; t < TH; t++) {
+                            if (valid[t] && cg < my_groups) {
+                                uint16_t *yp = s.y + (size_t)slot[t] * K + c0 + 16 * q;
 #pragma unroll
-                            for (int half = 0; half < 2; half++) {
-                                const v4f lo = acc[2 * half][t] * tw[t], hi = acc[2 * half + 1][t] * tw[t];
-                                v4i o;
-                                o.x = (int)pack_bf16x2(lo[0], lo[1]);
-                                o.y = (int)pack_bf16x2(lo[2], lo[3]);
-                                o.z = (int)pack_bf16x2(hi[0], hi[1]);
-                                o.w = (int)pack_bf16x2(hi[2], hi[3]);
-                                *reinterpret_cast<v4i *>(yp + 8 * half) = o;
+                                for (int half = 0; half < 2; half++) {
+                                    const v4f lo = acc[2 * half][t] * tw[t], hi = acc[2 * half + 1][t] * tw[t];
+                                    v4i o;
+                                    o.x = (int)pack_bf16x2(lo[0], lo[1]);
+                                    o.y = (int)pack_bf16x2(lo[2], lo[3]);
+                                    o.z = (int)pack_bf16x2(hi[0], hi[1]);
+                                    o.w = (int)pack_bf16x2(hi[2], hi[3]);
+                                    *reinterpret_cast<v4i *>(yp + 8 * half) = o;
+                                }
                             }
-                        }
 #pragma unroll
-                        for (int a = 0; a < 4; a++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+                            for (int a = 0; a < 4; a++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+                        }
+                        cib = 0;
+                        cg++;
                     }
-                    cib = 0;
-                    cg++;
                 }
             }
         }
+        wait_vmcnt<0>();
+    };
+
+    // ---- item loop ------------------------------------------------------------------------------------------------
+    // Queue qq holds row blocks [qq * per_q, ...) as items: the up/gate items of `lag` blocks first, then alternately
+    // the up/gate items of block lag + r and the down items of block r, at the end the down items of the last `lag`
+    // blocks.  A down item waits for the flags of its block's up/gate items, which are EARLIER in the same queue:
+    // whoever took them is running and waits for nothing later, so the queues drain with any number of resident
+    // workgroups.  A workgroup that finds its queue empty moves on to the next one.
+    auto blocks_of = [&](int qq) {
+        const int left = n_live - qq * per_q;
+        return left < 0 ? 0 : (left < per_q ? left : per_q);
+    };
+    int qq = blockIdx.x & 7, visited = 0;
+    while (true) {
+        if (tid == 0) {
+            int it = -1;
+            while (visited < 8) {
+                const int nb = blocks_of(qq);
+                const int idx = nb > 0 ? __hip_atomic_fetch_add(&s.ctl->tile_head[qq], 1, __ATOMIC_RELAXED,
+                                                                __HIP_MEMORY_SCOPE_AGENT)
+                                       : 0;
+                if (idx < nb * (per_up + per_down)) {
+                    it = idx;
+                    break;
+                }
+                qq = (qq + 1) & 7;
+                visited++;
+            }
+            s_item[0] = it;
+            s_item[1] = qq;
+        }
+        __syncthreads();
+        const int item = __builtin_amdgcn_readfirstlane(s_item[0]);
+        const int qi = __builtin_amdgcn_readfirstlane(s_item[1]);
+        if (item < 0) break;
+        const int nb = blocks_of(qi);
+        const int lag = s.lag < nb ? s.lag : nb;
+        const int head_items = lag * per_up, mid_items = (nb - lag) * (per_up + per_down);
+        int up = -1, down = -1;
+        if (item < head_items) {
+            up = item;
+        } else if (item < head_items + mid_items) {
+            const int i = item - head_items;
+            const int round = i / (per_up + per_down);
+            const int off = i - round * (per_up + per_down);
+            if (off < per_up)
+                up = (lag + round) * per_up + off;
+            else
+                down = round * per_down + (off - per_up);
+        } else {
+            down = (nb - lag) * per_down + (item - head_items - mid_items);
+        }
+        if (up >= 0)
+            up_item(qi * per_q + up / per_up, up % per_up);
+        else
+            down_item(qi * per_q + down / per_down, down % per_down);
+        __syncthreads();   // everybody is done with the item's LDS tables and rings before the next item refills them
     }
-    wait_vmcnt<0>();
+    if (tid == 0) {
+        const int left = __hip_atomic_fetch_add(&s.ctl->tile_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (left == (int)gridDim.x - 1) {
+            for (int i = 0; i < 8; i++) store_agent(&s.ctl->tile_head[i], 0);
+            store_agent(&s.ctl->tile_done, 0);
+        }
+    }
 }
 
 // out[t] = bf16(out[t] + sum over the token's live slots of y[slot]); the last workgroup to leave closes the epoch.
@@ -491,6 +612,12 @@ __global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams s
 
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
+int env_int(const char *name, int dflt)
+{
+    const char *e = getenv(name);
+    return e ? atoi(e) : dflt;
+}
+
 int tail_tiles(int n_ib) { return n_ib > kStages ? n_ib : kStages; }
 
 typedef void (*TileFn)(const TileParams);
@@ -510,14 +637,23 @@ TileFn pick(int th)
 
 }  // namespace
 
+// 64-column groups per DOWN item: about 14 ring steps (a step is one group x one slice), a multiple of 4 so that
+// every pair of wavefronts gets the same number of groups
+static int groups_per_item(int n_ib)
+{
+    const int e = env_int("ALPHA_MOE_TILE_GPS", 0);
+    if (e > 0) return (e + 3) / 4 * 4;
+    return 4 * ((14 + n_ib - 1) / n_ib);
+}
+
 bool tile_supported(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
 {
     (void)E;
-    (void)sorted_num;
     const int tm = 2 * tiles_per_wave(block_m);
     const int n_ib = N / 256;
+    const int64_t n_mb = ((int64_t)sorted_num + block_m - 1) / block_m;
     return n_ib <= kTileMaxIb && tail_tiles(n_ib) * tm * 2048 <= kMaxTailBytes && K <= 128 * kTileMaxKb &&
-           (K / 128) * n_ib <= kTileMaxW2s && (int64_t)M * top_k <= kMaxSlots;
+           (K / 128) * n_ib <= kTileMaxW2s && (int64_t)M * top_k <= kMaxSlots && n_mb * n_ib <= kMaxUnits;
 }
 
 size_t tile_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
@@ -526,7 +662,7 @@ size_t tile_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_nu
     const int tm = 2 * tiles_per_wave(block_m);
     const size_t n_mb = ((size_t)sorted_num + block_m - 1) / block_m;
     return align_up(kPrefixBytes) + align_up((size_t)M * top_k * K * sizeof(uint16_t)) +
-           align_up(n_mb * (N / 256) * tm * 2048);
+           align_up(n_mb * (N / 256) * tm * 2048) + align_up(n_mb * (N / 256) * tm * 16 * sizeof(float));
 }
 
 hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
@@ -534,20 +670,43 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
     uint8_t *ws = static_cast<uint8_t *>(workspace);
     TileParams s;
     s.p = p;
-    s.ctl = reinterpret_cast<StreamCtl *>(ws);
-    s.live = reinterpret_cast<int *>(ws + kOffLive);
-    s.y = reinterpret_cast<uint16_t *>(ws + align_up(kPrefixBytes));
-    s.aqs = ws + align_up(kPrefixBytes) + align_up((size_t)p.M * p.top_k * p.K * sizeof(uint16_t));
     s.n_ib = p.N / 256;
     s.nkb = p.K / 128;
     s.n_mb_max = (p.sorted_num + p.block_m - 1) / p.block_m;
     const int tm = 2 * tiles_per_wave(p.block_m);
+    size_t off = align_up(kPrefixBytes);
+    s.ctl = reinterpret_cast<StreamCtl *>(ws);
+    s.flag = reinterpret_cast<int *>(ws + kOffFlag);
+    s.live = reinterpret_cast<int *>(ws + kOffLive);
+    s.y = reinterpret_cast<uint16_t *>(ws + off);
+    off += align_up((size_t)p.M * p.top_k * p.K * sizeof(uint16_t));
+    s.aqs = ws + off;
+    off += align_up((size_t)s.n_mb_max * s.n_ib * tm * 2048);
+    s.sas = reinterpret_cast<float *>(ws + off);
+    s.gps = groups_per_item(s.n_ib);
+    s.n_cs = ((p.K >> 6) + s.gps - 1) / s.gps;
+    // up/gate items of this many row blocks run ahead of the first down items of a queue: with ~32 workgroups
+    // on a queue, a down item's up/gate items were taken at least two rounds of the queue earlier
+    s.lag = env_int("ALPHA_MOE_TILE_LAG", 64);
+    s.w_nt = env_int("ALPHA_MOE_TILE_NT", -1);
+    if (s.lag < 1) s.lag = 1;
     const TileFn fn = pick(tm / 2);
     const int lds_bytes = kARingBytes + tail_tiles(s.n_ib) * tm * 2048;
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          kARingBytes + kMaxTailBytes);
     if (err != hipSuccess) return err;
-    const int grid = (s.n_mb_max + 7) / 8 * 8;
+    // persistent workgroups, one per compute unit (the rings take most of a CU's LDS); fewer when there is less work
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            return 256;
+        return n;
+    }();
+    const int64_t items = (int64_t)s.n_mb_max * (s.n_ib + s.n_cs);
+    int grid = env_int("ALPHA_MOE_TILE_GRID", cus);
+    if (grid > items) grid = (int)((items + 7) / 8 * 8);
+    if (grid < 8) grid = 8;
     hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(512), lds_bytes, stream, s);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
@@ -559,12 +718,3 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
 }
 
 }  // namespace alpha_moe
-
-#ifdef ALPHA_MOE_TRACE
-extern "C" int alpha_moe_debug_tile_trace_read(void *dst)
-{
-    (void)hipDeviceSynchronize();
-    (void)hipMemcpyFromSymbol(dst, HIP_SYMBOL(alpha_moe::g_tile_trace), sizeof(alpha_moe::g_tile_trace));
-    return 1024 * alpha_moe::kTraceSteps;
-}
-#endif
