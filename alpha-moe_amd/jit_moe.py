@@ -95,7 +95,9 @@ def main(argv=None):
     w1_scale = (torch.randn((E, N // 128, K // 128), dtype=torch.float32) * 0.01).to(dev)
     w2_scale = (torch.randn((E, K // 128, N // 256), dtype=torch.float32) * 0.01).to(dev)
 
-    candidates = [(bm, bn, wn, st) for bm in args.block_ms for (bn, wn) in ((64, 4), (32, 8)) for st in args.stages]
+    # row blocks above 32 rows take the tile kernel, which ignores block_n, warp_n and stages: one candidate each
+    candidates = [(bm, bn, wn, st) for bm in args.block_ms if bm <= 32 for (bn, wn) in ((64, 4), (32, 8))
+                  for st in args.stages] + [(bm, 64, 4, 3) for bm in args.block_ms if bm > 32]
     times = {}
     for num_tokens in args.batch_sizes:
         times[num_tokens] = {c: [] for c in candidates}
