@@ -737,6 +737,8 @@ HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int bl
     // a DOWN item reads all n_ib slices of its columns: 2 KiB * n_ib per 16-column tile
     int64_t down_target = 256 << 10;
     if (mb_est * ((h.n_ct * 2048 * h.n_ib + down_target - 1) / down_target) < cus / 2) down_target = 128 << 10;
+    // small experts, about a row block per compute unit: one DOWN item per block (Qwen3-Next shard, M = 32: -7 %)
+    if ((int64_t)h.n_ct * 2048 * h.n_ib <= (512 << 10) && mb_est * 4 >= cus * 3) down_target = 512 << 10;
     int tpi = (int)(down_target / (2048 * h.n_ib)) / 16 * 16;
     tpi = env_int("ALPHA_MOE_TPI", tpi);
     if (tpi < 16) tpi = 16;
