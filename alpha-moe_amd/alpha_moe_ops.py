@@ -15,6 +15,13 @@ def _fused_moe_w8a8_up_down_fake(x, x_scale, w, w_scale, w2, w2_scale, sorted_to
     return None
 
 
+@torch.library.register_fake("alpha_moe::fused_moe_w8a8_up_down_store")
+def _fused_moe_w8a8_up_down_store_fake(x, x_scale, w, w_scale, w2, w2_scale, sorted_token_ids, expert_ids,
+                                       num_tokens_post_padded, topk_weights, out, top_k, block_m, block_n, warp_n,
+                                       stages, scaling_factor):
+    return None
+
+
 @torch.library.register_fake("alpha_moe::per_token_group_quant_fp8")
 def _per_token_group_quant_fp8_fake(x, group_size):
     return (torch.empty_like(x, dtype=torch.float8_e4m3fn),
@@ -62,4 +69,16 @@ def fused_moe_w8a8_up_down(
     return out
 
 
-__all__ = ["fused_moe_w8a8_up_down"]
+def fused_moe_w8a8_up_down_store(x, x_scale, w, w_scale, w2, w2_scale, sorted_token_ids, expert_ids,
+                                 num_tokens_post_padded, topk_weights, out, top_k, block_m, block_n, warp_n, stages,
+                                 scaling_factor) -> torch.Tensor:
+    """``fused_moe_w8a8_up_down`` with store semantics: ``out`` is overwritten with the result, so it may come from
+    ``torch.empty_like`` and the zero-fill before every call (one more kernel launch at decode sizes) goes away.  The
+    reference has no such variant.  Returns ``out``."""
+    torch.ops.alpha_moe.fused_moe_w8a8_up_down_store(
+        x, x_scale, w, w_scale, w2, w2_scale, sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights, out,
+        top_k, block_m, block_n, warp_n, stages, scaling_factor)
+    return out
+
+
+__all__ = ["fused_moe_w8a8_up_down", "fused_moe_w8a8_up_down_store"]

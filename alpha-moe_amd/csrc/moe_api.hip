@@ -72,14 +72,13 @@ extern "C" size_t alpha_moe_workspace_bytes(int top_k, int M, int K, int N, int 
     return m > tile ? m : tile;
 }
 
-extern "C" int alpha_moe_fused_moe_w8a8_up_down(const uint8_t *x, const float *x_scale, const uint8_t *w,
-                                                const float *w_scale, const uint8_t *w2, const float *w2_scale,
-                                                uint16_t *out, const int32_t *sorted_token_ids,
-                                                const int32_t *expert_ids, const int32_t *num_tokens_post_padded,
-                                                const float *topk_weights, int top_k, int M, int K, int N,
-                                                int num_experts, int sorted_num, int block_m, int block_n, int warp_n,
-                                                int stages, float scaling_factor, void *workspace,
-                                                size_t workspace_bytes, void *stream)
+namespace {
+
+int run_fused_moe(const uint8_t *x, const float *x_scale, const uint8_t *w, const float *w_scale, const uint8_t *w2,
+                  const float *w2_scale, uint16_t *out, const int32_t *sorted_token_ids, const int32_t *expert_ids,
+                  const int32_t *num_tokens_post_padded, const float *topk_weights, int top_k, int M, int K, int N,
+                  int num_experts, int sorted_num, int block_m, int block_n, int warp_n, int stages,
+                  float scaling_factor, void *workspace, size_t workspace_bytes, void *stream, int overwrite)
 {
     if (!x || !x_scale || !w || !w_scale || !w2 || !w2_scale || !out || !sorted_token_ids || !expert_ids ||
         !num_tokens_post_padded || !topk_weights)
@@ -98,6 +97,7 @@ extern "C" int alpha_moe_fused_moe_w8a8_up_down(const uint8_t *x, const float *x
     p.topk_w = topk_weights;
     p.top_k = top_k; p.M = M; p.K = K; p.N = N; p.E = num_experts; p.sorted_num = sorted_num; p.block_m = block_m;
     p.scaling = scaling_factor;
+    p.overwrite = overwrite;
 
     hipStream_t hs = static_cast<hipStream_t>(stream);
     hipError_t err;
@@ -112,6 +112,37 @@ extern "C" int alpha_moe_fused_moe_w8a8_up_down(const uint8_t *x, const float *x
         if (err == hipSuccess) err = launch_finalize(p, hs);
     }
     return err == hipSuccess ? ALPHA_MOE_OK : ALPHA_MOE_ERR_LAUNCH;
+}
+
+}  // namespace
+
+extern "C" int alpha_moe_fused_moe_w8a8_up_down(const uint8_t *x, const float *x_scale, const uint8_t *w,
+                                                const float *w_scale, const uint8_t *w2, const float *w2_scale,
+                                                uint16_t *out, const int32_t *sorted_token_ids,
+                                                const int32_t *expert_ids, const int32_t *num_tokens_post_padded,
+                                                const float *topk_weights, int top_k, int M, int K, int N,
+                                                int num_experts, int sorted_num, int block_m, int block_n, int warp_n,
+                                                int stages, float scaling_factor, void *workspace,
+                                                size_t workspace_bytes, void *stream)
+{
+    return run_fused_moe(x, x_scale, w, w_scale, w2, w2_scale, out, sorted_token_ids, expert_ids,
+                         num_tokens_post_padded, topk_weights, top_k, M, K, N, num_experts, sorted_num, block_m, block_n,
+                         warp_n, stages, scaling_factor, workspace, workspace_bytes, stream, 0);
+}
+
+extern "C" int alpha_moe_fused_moe_w8a8_up_down_store(const uint8_t *x, const float *x_scale, const uint8_t *w,
+                                                      const float *w_scale, const uint8_t *w2, const float *w2_scale,
+                                                      uint16_t *out, const int32_t *sorted_token_ids,
+                                                      const int32_t *expert_ids,
+                                                      const int32_t *num_tokens_post_padded, const float *topk_weights,
+                                                      int top_k, int M, int K, int N, int num_experts, int sorted_num,
+                                                      int block_m, int block_n, int warp_n, int stages,
+                                                      float scaling_factor, void *workspace, size_t workspace_bytes,
+                                                      void *stream)
+{
+    return run_fused_moe(x, x_scale, w, w_scale, w2, w2_scale, out, sorted_token_ids, expert_ids,
+                         num_tokens_post_padded, topk_weights, top_k, M, K, N, num_experts, sorted_num, block_m, block_n,
+                         warp_n, stages, scaling_factor, workspace, workspace_bytes, stream, 1);
 }
 
 extern "C" const char *alpha_moe_status_string(int status)

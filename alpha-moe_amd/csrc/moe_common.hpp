@@ -43,6 +43,7 @@ struct MoeParams {
     const float *topk_w;
     int top_k, M, K, N, E, sorted_num, block_m;
     float scaling;
+    int overwrite;              // 1: out = bf16(sum), whatever out held; 0: out = bf16(out + sum)
 };
 
 __device__ __forceinline__ v4i ldg128(const uint8_t *p) { return *reinterpret_cast<const v4i *>(p); }
@@ -128,7 +129,7 @@ constexpr size_t kPrefixBytes = kOffLive + sizeof(int) * kMaxSlots;
 // rounds the sums into p.out.
 hipError_t launch_zero_acc(const MoeParams &p, hipStream_t stream);
 hipError_t launch_direct(const MoeParams &p, int warp_n, int stages, hipStream_t stream);
-hipError_t launch_finalize(const MoeParams &p, hipStream_t stream);   // out = bf16(out + acc)
+hipError_t launch_finalize(const MoeParams &p, hipStream_t stream);   // out = bf16(out + acc), or bf16(acc)
 
 // Persistent work-queue kernel for decode-sized batches (block_m <= 32 and bounded sizes): split-K up items ->
 // SwiGLU/requant -> column-slab down items -> per-token reduction, chained through counters in the workspace.

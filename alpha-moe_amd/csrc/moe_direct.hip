@@ -257,13 +257,16 @@ __global__ __launch_bounds__(256) void moe_zero_kernel(float *__restrict__ acc, 
     if (i < n4) reinterpret_cast<v4f *>(acc)[i] = (v4f){0.f, 0.f, 0.f, 0.f};
 }
 
-// out[i] = bf16(float(out[i]) + acc[i]).  n4 = M*K/4 (K % 128 == 0, so rows never straddle).
-__global__ __launch_bounds__(256) void moe_finalize_kernel(float *__restrict__ acc, uint16_t *__restrict__ out, int n4)
+// out[i] = bf16(float(out[i]) + acc[i]), or bf16(acc[i]) when overwriting.  n4 = M*K/4 (K % 128 == 0, so rows never
+// straddle).
+__global__ __launch_bounds__(256) void moe_finalize_kernel(float *__restrict__ acc, uint16_t *__restrict__ out, int n4,
+                                                           int overwrite)
 {
     const int i = blockIdx.x * 256 + threadIdx.x;
     if (i >= n4) return;
     v4f a = reinterpret_cast<v4f *>(acc)[i];
-    uint2 o = reinterpret_cast<uint2 *>(out)[i];
+    uint2 o = {0u, 0u};
+    if (!overwrite) o = reinterpret_cast<uint2 *>(out)[i];
     const float o0 = __builtin_bit_cast(float, o.x << 16), o1 = __builtin_bit_cast(float, o.x & 0xffff0000u);
     const float o2 = __builtin_bit_cast(float, o.y << 16), o3 = __builtin_bit_cast(float, o.y & 0xffff0000u);
     o.x = pack_bf16x2(o0 + a[0], o1 + a[1]);
@@ -333,7 +336,8 @@ hipError_t launch_zero_acc(const MoeParams &p, hipStream_t stream)
 hipError_t launch_finalize(const MoeParams &p, hipStream_t stream)
 {
     const int n4 = (int)((int64_t)p.M * p.K / 4);
-    hipLaunchKernelGGL(moe_finalize_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, p.acc, p.out, n4);
+    hipLaunchKernelGGL(moe_finalize_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, stream, p.acc, p.out, n4,
+                       p.overwrite);
     return hipGetLastError();
 }
 

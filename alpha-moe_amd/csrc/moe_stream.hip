@@ -600,7 +600,8 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 for (int k = 0; k < 8; k++) sum += __builtin_bit_cast(v4f, bits[k]);
             }
             uint2 *op = reinterpret_cast<uint2 *>(p.out + (size_t)t * K + c);
-            uint2 o = *op;
+            uint2 o = {0u, 0u};
+            if (!p.overwrite) o = *op;
             const float o0 = __builtin_bit_cast(float, o.x << 16), o1 = __builtin_bit_cast(float, o.x & 0xffff0000u);
             const float o2 = __builtin_bit_cast(float, o.y << 16), o3 = __builtin_bit_cast(float, o.y & 0xffff0000u);
             o.x = pack_bf16x2(o0 + sum[0], o1 + sum[1]);

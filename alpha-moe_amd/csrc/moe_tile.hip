@@ -579,7 +579,8 @@ __global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams s
             }
         };
         v4i *op = reinterpret_cast<v4i *>(p.out + (size_t)t * p.K + c);
-        const v4i prior = *op;
+        v4i prior = {0, 0, 0, 0};
+        if (!p.overwrite) prior = *op;
         const int *live = s.live + t * p.top_k;
         const uint16_t *yrow = s.y + (size_t)t * p.top_k * p.K + c;
         for (int s0 = 0; s0 < p.top_k; s0 += 8) {   // slot order: the sum depends on nothing but the inputs

@@ -46,12 +46,11 @@ void check_tensor(const at::Tensor &t, const char *name, at::ScalarType dtype, c
     TORCH_CHECK(t.is_contiguous(), name, " must be contiguous");
 }
 
-void fused_moe_w8a8_up_down(const at::Tensor &x, const at::Tensor &x_scale, const at::Tensor &w,
-                            const at::Tensor &w_scale, const at::Tensor &w2, const at::Tensor &w2_scale,
-                            const at::Tensor &sorted_token_ids, const at::Tensor &expert_ids,
-                            const at::Tensor &num_tokens_post_padded, const at::Tensor &topk_weights,
-                            at::Tensor &out, int64_t top_k, int64_t block_m, int64_t block_n, int64_t warp_n,
-                            int64_t stages, double scaling_factor)
+void run_fused_moe(const at::Tensor &x, const at::Tensor &x_scale, const at::Tensor &w, const at::Tensor &w_scale,
+                   const at::Tensor &w2, const at::Tensor &w2_scale, const at::Tensor &sorted_token_ids,
+                   const at::Tensor &expert_ids, const at::Tensor &num_tokens_post_padded,
+                   const at::Tensor &topk_weights, at::Tensor &out, int64_t top_k, int64_t block_m, int64_t block_n,
+                   int64_t warp_n, int64_t stages, double scaling_factor, bool store)
 {
     TORCH_CHECK(x.is_cuda(), "x must be a GPU tensor");
     const at::Device dev = x.device();
@@ -98,7 +97,8 @@ void fused_moe_w8a8_up_down(const at::Tensor &x, const at::Tensor &x_scale, cons
                                   static_cast<int>(E), static_cast<int>(sorted_num), static_cast<int>(block_m));
     at::Tensor ws = workspace_for(dev, stream, ws_bytes);
 
-    const int rc = alpha_moe_fused_moe_w8a8_up_down(
+    const auto entry = store ? alpha_moe_fused_moe_w8a8_up_down_store : alpha_moe_fused_moe_w8a8_up_down;
+    const int rc = entry(
         static_cast<const uint8_t *>(x.const_data_ptr()), x_scale.const_data_ptr<float>(),
         static_cast<const uint8_t *>(w.const_data_ptr()), w_scale.const_data_ptr<float>(),
         static_cast<const uint8_t *>(w2.const_data_ptr()), w2_scale.const_data_ptr<float>(),
@@ -110,6 +110,29 @@ void fused_moe_w8a8_up_down(const at::Tensor &x, const at::Tensor &x_scale, cons
         static_cast<float>(scaling_factor), ws.data_ptr(), static_cast<size_t>(ws.numel()),
         static_cast<void *>(stream));
     TORCH_CHECK(rc == ALPHA_MOE_OK, "alpha_moe_fused_moe_w8a8_up_down failed: ", alpha_moe_status_string(rc));
+}
+
+void fused_moe_w8a8_up_down(const at::Tensor &x, const at::Tensor &x_scale, const at::Tensor &w,
+                            const at::Tensor &w_scale, const at::Tensor &w2, const at::Tensor &w2_scale,
+                            const at::Tensor &sorted_token_ids, const at::Tensor &expert_ids,
+                            const at::Tensor &num_tokens_post_padded, const at::Tensor &topk_weights,
+                            at::Tensor &out, int64_t top_k, int64_t block_m, int64_t block_n, int64_t warp_n,
+                            int64_t stages, double scaling_factor)
+{
+    run_fused_moe(x, x_scale, w, w_scale, w2, w2_scale, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                  topk_weights, out, top_k, block_m, block_n, warp_n, stages, scaling_factor, false);
+}
+
+// Store semantics: out = bf16(sum) whatever it held, so the caller need not zero-fill it first.
+void fused_moe_w8a8_up_down_store(const at::Tensor &x, const at::Tensor &x_scale, const at::Tensor &w,
+                                  const at::Tensor &w_scale, const at::Tensor &w2, const at::Tensor &w2_scale,
+                                  const at::Tensor &sorted_token_ids, const at::Tensor &expert_ids,
+                                  const at::Tensor &num_tokens_post_padded, const at::Tensor &topk_weights,
+                                  at::Tensor &out, int64_t top_k, int64_t block_m, int64_t block_n, int64_t warp_n,
+                                  int64_t stages, double scaling_factor)
+{
+    run_fused_moe(x, x_scale, w, w_scale, w2, w2_scale, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                  topk_weights, out, top_k, block_m, block_n, warp_n, stages, scaling_factor, true);
 }
 
 // (q, scale) = per_token_group_quant_fp8(x, 128): what the reference's callers get from SGLang (jit_moe.py:142).
@@ -176,4 +199,10 @@ TORCH_LIBRARY_FRAGMENT(alpha_moe, m)
           ") -> ()");
     // GPU tensors of PyTorch-ROCm carry the dispatch key named CUDA
     m.impl("fused_moe_w8a8_up_down", c10::DispatchKey::CUDA, &fused_moe_w8a8_up_down);
+    m.def("fused_moe_w8a8_up_down_store("
+          "Tensor x, Tensor x_scale, Tensor w, Tensor w_scale, Tensor w2, Tensor w2_scale, "
+          "Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_post_padded, Tensor topk_weights, "
+          "Tensor(a!) out, int top_k, int block_m, int block_n, int warp_n, int stages, float scaling_factor"
+          ") -> ()");
+    m.impl("fused_moe_w8a8_up_down_store", c10::DispatchKey::CUDA, &fused_moe_w8a8_up_down_store);
 }

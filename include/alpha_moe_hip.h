@@ -67,7 +67,25 @@ int alpha_moe_fused_moe_w8a8_up_down(
     int block_m, int block_n, int warp_n, int stages,
     float scaling_factor, void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
 
-/* Bytes of scratch the call above needs for these sizes (0 if any is not positive). */
+/*
+ * The same call with store semantics: out = bf16(sum), whatever `out` held before, so the caller's zero-fill of
+ * `out` (README.md:49,62 and extra/sglang.patch:31 of the reference: `torch.zeros_like(hidden_states)` before every
+ * call) and its launch are not needed.  Every element of out[0:M, 0:K] is written, also for tokens none of whose
+ * slots is live.  Same arguments, checks, workspace and status codes as alpha_moe_fused_moe_w8a8_up_down.
+ * The reference has no such variant: its kernel can only add, because top_k * I/128 workgroups contribute to a row.
+ */
+int alpha_moe_fused_moe_w8a8_up_down_store(
+    const uint8_t *x, const float *x_scale,
+    const uint8_t *w, const float *w_scale,
+    const uint8_t *w2, const float *w2_scale,
+    uint16_t *out,
+    const int32_t *sorted_token_ids, const int32_t *expert_ids, const int32_t *num_tokens_post_padded,
+    const float *topk_weights,
+    int top_k, int M, int K, int N, int num_experts, int sorted_num,
+    int block_m, int block_n, int warp_n, int stages,
+    float scaling_factor, void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
+
+/* Bytes of scratch the calls above need for these sizes (0 if any is not positive). */
 size_t alpha_moe_workspace_bytes(int top_k, int M, int K, int N, int num_experts, int sorted_num, int block_m);
 
 /*

@@ -10,7 +10,7 @@ MAX_ABS_OVER_MAX_REF = 1e-2
 MIN_COSINE = 0.9999
 
 
-def run_op(P, block_m, block_n, warp_n, stages, out=None, scaling=None, via="torch", workspace=None):
+def run_op(P, block_m, block_n, warp_n, stages, out=None, scaling=None, via="torch", workspace=None, store=False):
     import alpha_moe
     W = P.weights
     s_ids, e_ids, total = P.align(block_m)
@@ -18,7 +18,8 @@ def run_op(P, block_m, block_n, warp_n, stages, out=None, scaling=None, via="tor
         out = torch.zeros((P.M, P.shape.K), dtype=torch.bfloat16, device=P.x.device)
     scaling = P.shape.scaling_factor if scaling is None else scaling
     if via == "torch":
-        torch.ops.alpha_moe.fused_moe_w8a8_up_down(P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids,
+        op = torch.ops.alpha_moe.fused_moe_w8a8_up_down_store if store else torch.ops.alpha_moe.fused_moe_w8a8_up_down
+        op(P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids,
                                                    total, P.topk_weights, out, P.shape.top_k, block_m, block_n, warp_n,
                                                    stages, scaling)
     else:
@@ -26,7 +27,9 @@ def run_op(P, block_m, block_n, warp_n, stages, out=None, scaling=None, via="tor
         ws_bytes = alpha_moe.c_abi.alpha_moe_workspace_bytes(P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E, s_ids.numel(), block_m)
         ws = workspace if workspace is not None else torch.zeros(ws_bytes, dtype=torch.uint8, device=P.x.device)
         assert ws.numel() >= ws_bytes
-        rc = alpha_moe.c_abi.alpha_moe_fused_moe_w8a8_up_down(
+        entry = (alpha_moe.c_abi.alpha_moe_fused_moe_w8a8_up_down_store if store
+                 else alpha_moe.c_abi.alpha_moe_fused_moe_w8a8_up_down)
+        rc = entry(
             P.x.data_ptr(), P.x_scale.data_ptr(), W.w1.data_ptr(), W.w1_scale.data_ptr(), W.w2.data_ptr(),
             W.w2_scale.data_ptr(), out.data_ptr(), s_ids.data_ptr(), e_ids.data_ptr(), total.data_ptr(),
             P.topk_weights.data_ptr(), P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E, s_ids.numel(), block_m,

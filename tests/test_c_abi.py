@@ -81,6 +81,14 @@ def test_null_pointers_and_small_workspace_are_refused_without_touching_a_device
                                                 ctypes.c_void_p(4096), 1024, None) == 7
     assert lib.alpha_moe_fused_moe_w8a8_up_down(*fake, 9, 64, 7168, 512, 257, 4431, 12, 64, 4, 3, 2.5,
                                                 ctypes.c_void_p(4096), 1 << 40, None) == 3
+    # the store variant runs the same checks
+    lib.alpha_moe_fused_moe_w8a8_up_down_store.restype = ctypes.c_int
+    lib.alpha_moe_fused_moe_w8a8_up_down_store.argtypes = lib.alpha_moe_fused_moe_w8a8_up_down.argtypes
+    assert lib.alpha_moe_fused_moe_w8a8_up_down_store(*args) == 1
+    assert lib.alpha_moe_fused_moe_w8a8_up_down_store(*fake, 9, 64, 7168, 512, 257, 4431, 16, 64, 4, 3, 2.5, None, 0,
+                                                      None) == 7
+    assert lib.alpha_moe_fused_moe_w8a8_up_down_store(*fake, 9, 64, 7168, 512, 257, 4431, 12, 64, 4, 3, 2.5,
+                                                      ctypes.c_void_p(4096), 1 << 40, None) == 3
 
 
 def test_workspace_bytes_is_monotone_and_covers_both_kernel_families(lib):

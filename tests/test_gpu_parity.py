@@ -61,6 +61,39 @@ def test_add_semantics_scaling_and_zero_weights(c1):
     P.topk_weights = saved
 
 
+@pytest.mark.parametrize("knobs", [(16, 32, 8, 2), (16, 64, 4, 5), (64, 64, 4, 3), (128, 64, 4, 3)])
+def test_store_variant_overwrites_whatever_out_held(c1, knobs):
+    """fused_moe_w8a8_up_down_store: out = bf16(sum) on every element, NaN-filled or not, and bit for bit what the
+    adding call leaves in a zero-filled out - streaming and tile kernels, torch op and C ABI."""
+    P, ref = c1
+    zero = run_op(P, *knobs, via="c_abi")
+    assert_parity(zero, ref, f"knobs {knobs}")
+    for via in ("torch", "c_abi"):
+        junk = torch.full((P.M, P.shape.K), float("nan"), dtype=torch.bfloat16, device=DEV)
+        got = run_op(P, *knobs, out=junk, via=via, store=True)
+        assert torch.equal(got, zero), (knobs, via)
+    # a token none of whose slots contributes still gets its row written
+    saved = P.topk_weights
+    P.topk_weights = torch.zeros_like(saved)
+    junk = torch.full((P.M, P.shape.K), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert float(run_op(P, *knobs, out=junk, store=True).float().abs().max()) == 0.0
+    P.topk_weights = saved
+
+
+def test_store_variant_fallback_kernel():
+    """Six 128-column slices with 128-row blocks exceed the tile kernel's LDS budget: the fallback kernel serves the call,
+    and its store variant overwrites too."""
+    from alpha_moe_python.workloads import Shape
+    shape = Shape("fb", E=6, top_k=2, K=256, I=768, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0)
+    W = make_weights(shape, device=DEV, seed=5)
+    P = make_problem(W, 150, seed=5)
+    ref = oracle_out(P)
+    assert_parity(run_op(P, 128, 64, 4, 2, via="c_abi"), ref, "fallback kernel")
+    junk = torch.full((P.M, P.shape.K), float("nan"), dtype=torch.bfloat16, device=DEV)
+    # this kernel sums with fp32 atomics, so two runs agree to rounding, not bit for bit
+    assert_parity(run_op(P, 128, 64, 4, 2, out=junk, via="c_abi", store=True), ref, "fallback kernel, store")
+
+
 @pytest.mark.parametrize("M,E,top_k,K,I", [(1, 4, 2, 128, 128), (3, 5, 3, 384, 256), (37, 3, 2, 256, 384), (200, 2, 1, 128, 128)])
 def test_ragged_small_shapes(M, E, top_k, K, I):
     """K a single block, K % 256 == 128 (the reference silently drops the last 128 columns there), more I blocks,
