@@ -145,6 +145,8 @@ extern "C" int alpha_moe_fused_moe_w8a8_up_down_store(const uint8_t *x, const fl
                          warp_n, stages, scaling_factor, workspace, workspace_bytes, stream, 1);
 }
 
+extern "C" size_t alpha_moe_workspace_zero_bytes(void) { return (stream_prefix_bytes() + 255) & ~(size_t)255; }
+
 extern "C" const char *alpha_moe_status_string(int status)
 {
     switch (status) {

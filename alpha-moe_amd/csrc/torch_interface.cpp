@@ -33,7 +33,10 @@ at::Tensor workspace_for(const at::Device &dev, hipStream_t stream, size_t bytes
     if (!slot.defined() || static_cast<size_t>(slot.numel()) < bytes) {
         size_t cap = 1 << 20;
         while (cap < bytes) cap <<= 1;
-        slot = at::zeros({static_cast<int64_t>(cap)}, at::TensorOptions().dtype(at::kByte).device(dev));
+        slot = at::empty({static_cast<int64_t>(cap)}, at::TensorOptions().dtype(at::kByte).device(dev));
+        // only the control block, counters and flags have to start at zero (1.5 MiB, not the whole buffer: under HIP
+        // graph capture this fill is recorded and runs on every replay)
+        slot.narrow(0, 0, static_cast<int64_t>(alpha_moe_workspace_zero_bytes())).zero_();
     }
     return slot;
 }

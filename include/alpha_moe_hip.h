@@ -51,7 +51,8 @@ enum alpha_moe_status {
  *   (block_n, warp_n) (64,4) or (32,8) wavefronts per workgroup = warp_n, w1 rows per wavefront = block_n
  *   stages           1..5              K-blocks of loads kept in flight per wavefront
  *   workspace        device scratch of at least alpha_moe_workspace_bytes(top_k, M, K, N, num_experts, sorted_num,
- *                    block_m) bytes, 256-byte aligned.  It must be ZERO-FILLED once, before its first use; after
+ *                    block_m) bytes, 256-byte aligned.  Its first alpha_moe_workspace_zero_bytes() bytes must be
+ *                    ZERO-FILLED once, before its first use (zero-filling all of it is fine too); after
  *                    that its contents belong to the library (self-resetting counters, per-launch epochs) and the
  *                    same buffer serves any number of calls, of any sizes it is large enough for, without being
  *                    cleared.  Calls that share a workspace must be ordered on one stream.
@@ -87,6 +88,13 @@ int alpha_moe_fused_moe_w8a8_up_down_store(
 
 /* Bytes of scratch the calls above need for these sizes (0 if any is not positive). */
 size_t alpha_moe_workspace_bytes(int top_k, int M, int K, int N, int num_experts, int sorted_num, int block_m);
+
+/*
+ * How many bytes at the start of a workspace have to be zero before its first use (the control block, counters and
+ * flags; independent of the problem size).  The rest may hold anything.  No counterpart in the reference, which has
+ * no scratch memory.
+ */
+size_t alpha_moe_workspace_zero_bytes(void);
 
 /*
  * The argument checks of the call above without touching the device: returns the status the launch would

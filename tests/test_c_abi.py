@@ -91,6 +91,14 @@ def test_null_pointers_and_small_workspace_are_refused_without_touching_a_device
                                                       ctypes.c_void_p(4096), 1 << 40, None) == 3
 
 
+def test_zeroed_prefix_is_small_and_inside_every_workspace(lib):
+    lib.alpha_moe_workspace_zero_bytes.restype = ctypes.c_size_t
+    lib.alpha_moe_workspace_zero_bytes.argtypes = []
+    z = lib.alpha_moe_workspace_zero_bytes()
+    assert z > 0 and z % 256 == 0 and z <= 4 << 20
+    assert z <= lib.alpha_moe_workspace_bytes(2, 1, 128, 256, 1, 16, 16)
+
+
 def test_workspace_bytes_is_monotone_and_covers_both_kernel_families(lib):
     small = lib.alpha_moe_workspace_bytes(9, 1, 7168, 512, 257, 9 + 257 * 15, 16)
     big = lib.alpha_moe_workspace_bytes(9, 64, 7168, 512, 257, 576 + 257 * 15, 16)

@@ -302,3 +302,62 @@ def test_tile_kernel_result_independent_of_item_schedule(monkeypatch):
                     mp.setenv(k, v)
                 got = run_op(P, block_m, 64, 4, 3, via="c_abi")
             assert torch.equal(got, base), (block_m, env)
+
+
+@pytest.mark.parametrize("knobs", [(16, 32, 8, 5), (64, 64, 4, 3)])
+def test_workspace_needs_only_its_prefix_zeroed(c1, knobs):
+    """Everything behind alpha_moe_workspace_zero_bytes() may hold anything: fill it with 0xff."""
+    import alpha_moe
+    P, ref = c1
+    s_ids, _, _ = P.align(knobs[0])
+    need = alpha_moe.c_abi.alpha_moe_workspace_bytes(P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E, s_ids.numel(),
+                                                     knobs[0])
+    ws = torch.full((need,), 255, dtype=torch.uint8, device=DEV)
+    ws[: alpha_moe.c_abi.alpha_moe_workspace_zero_bytes()] = 0
+    first = run_op(P, *knobs, via="c_abi", workspace=ws)
+    assert_parity(first, ref, f"knobs {knobs}")
+    assert torch.equal(first, run_op(P, *knobs, via="c_abi", workspace=ws))
+
+
+@pytest.mark.parametrize("knobs,store", [((16, 32, 8, 5), False), ((16, 64, 4, 2), True), ((64, 64, 4, 3), False)])
+def test_hip_graph_capture_and_replay(c1, knobs, store):
+    """The operator allocates and synchronises nothing once it has run on a stream, so it can be captured into a HIP
+    graph there.  Replays with new activations in the captured buffers agree bit for bit with eager calls, with eager
+    work and synchronisations between the replays."""
+    from alpha_moe_python.workloads import Problem
+    P, _ = c1
+    W = P.weights
+    block_m = knobs[0]
+    s_ids, e_ids, total = P.align(block_m)
+    op = torch.ops.alpha_moe.fused_moe_w8a8_up_down_store if store else torch.ops.alpha_moe.fused_moe_w8a8_up_down
+    x, xs, tw = P.x.clone(), P.x_scale.clone(), P.topk_weights.clone()
+    out = torch.zeros((P.M, P.shape.K), dtype=torch.bfloat16, device=DEV)
+
+    def step():
+        if not store:
+            out.zero_()
+        op(x, xs, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids, total, tw, out, P.shape.top_k, *knobs,
+           P.shape.scaling_factor)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()   # first call on this stream: scratch is allocated and its prefix zeroed here, outside the capture
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for rep in range(4):
+        P2 = make_problem(W, P.M, seed=100 + rep)
+        # new activations and routing weights, same routing (the captured sorted ids): copy into the captured buffers
+        x.copy_(P2.x)
+        xs.copy_(P2.x_scale)
+        tw.copy_(P2.topk_weights)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        eager_problem = Problem(W, P.M, P2.x, P2.x_scale, P.topk_ids, P2.topk_weights)
+        want = run_op(eager_problem, *knobs, via="c_abi")   # eager work between replays
+        assert torch.equal(got, want), (knobs, store, rep)
