@@ -35,6 +35,8 @@
 // weights of experts that have a single block.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "moe_common.hpp"
 
 namespace alpha_moe {
@@ -56,7 +58,8 @@ struct TileParams {
     uint8_t *aqs;     // [row blocks][n_ib][TM] requantised operand tiles of 2 KiB
     float *sas;       // [row blocks][n_ib][TM * 16] their per-token scales
     int n_ib, nkb, n_mb_max;
-    int gps, n_cs;    // 64-column groups per DOWN item, DOWN items per row block
+    int gps, n_cs;    // 64-column groups per DOWN item, column slabs per row block
+    int nh;           // token parts per column slab (a DOWN item is one part of one slab)
     int lag;          // row blocks whose up/gate items precede the first down items of a queue
     int w_nt;         // weights with non-temporal loads: 1 always, 0 never, -1 for experts with a single row block
 };
@@ -222,7 +225,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
     int n_live = (__builtin_amdgcn_readfirstlane(p.ntpp[0]) + p.block_m - 1) / p.block_m;
     n_live = n_live < s.n_mb_max ? n_live : s.n_mb_max;
     const int per_q = (n_live + 7) >> 3;
-    const int per_up = n_ib, per_down = s.n_cs;
+    const int per_up = n_ib, per_down = s.n_cs * s.nh;
 
     // operand fragment of lane (n, q): chunks q and q+4 of row n; chunk c of row r sits at position c ^ ((r >> 1) & 7)
     const int f_n = (n >> 1) & 7;
@@ -365,21 +368,26 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         if (tid == 0) store_agent(&s.flag[unit], epoch);
     };
 
-    // ---- DOWN item: column groups [cs * gps, (cs + 1) * gps) of row block mb, all slices ------------------------------
+    // ---- DOWN item: column groups [cs * gps, (cs + 1) * gps) of row block mb, all slices, token part `part` ------------
     // 64 output columns per step group.  Pair w takes the slab's groups w, w + 4, ...; its two wavefronts split the
     // tokens as before and each loads two of the four w2 tiles of a step.  Matrix row r of tile k is output column
     // c0 + 16 (r / 4) + 4 k + r % 4, so lane (n, q) collects columns c0 + 16 q .. c0 + 16 q + 15 of token n over the
     // four tiles.  Load h of a tile: rows 8h + lane / 8.
-    auto down_item = [&](int mb, int cs) {
+    // The requantised tiles of ALL slices have to sit in LDS next to the weight ring.  Where I/128 slices of a whole
+    // block do not fit, the block's token tiles are served in TH / THD parts, each by an item of its own with THD
+    // tiles per wavefront: part `part` covers token tiles [part * 2 THD, (part + 1) * 2 THD).
+    auto down_item = [&](int mb, int cs, int part, auto thd_c) {
+        constexpr int THD = decltype(thd_c)::value;
+        constexpr int TMD = 2 * THD;
         const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
         if (e < 0 || e >= p.E) return;
         const bool nt = lone_block(mb, e);
-        int slot[TH];
-        bool valid[TH];
-        float tw[TH];
+        int slot[THD];
+        bool valid[THD];
+        float tw[THD];
 #pragma unroll
-        for (int t = 0; t < TH; t++) {
-            const int row = (g * TH + t) * 16 + n;
+        for (int t = 0; t < THD; t++) {
+            const int row = (part * TMD + g * THD + t) * 16 + n;
             const int idx = mb * p.block_m + row;
             int id = -1;
             if (row < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
@@ -430,24 +438,28 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         if (tid == 0)
             for (int ib = 0; ib < n_ib; ib++) tile_spin_until_ge(&s.flag[mb * n_ib + ib], epoch, s.ctl);
         __syncthreads();
-        // the requantised tiles and their scales come from scratch into LDS
+        // the requantised tiles of this part and their scales come from scratch into LDS: [slice][tile of the part]
         uint8_t *aq = xbuf;
-        for (int i = wave; i < n_ib * TM; i += 8) {
-            const uint8_t *src = s.aqs + ((size_t)mb * n_ib * TM + i) * 2048 + lane * 16;
+        for (int i = wave; i < n_ib * TMD; i += 8) {
+            const int ib = i / TMD, tt = i - ib * TMD;
+            const uint8_t *src = s.aqs + ((size_t)(mb * n_ib + ib) * TM + part * TMD + tt) * 2048 + lane * 16;
             dma16_agent(src, aq + i * 2048);
             dma16_agent(src + 1024, aq + i * 2048 + 1024);
         }
-        for (int i = tid; i < n_ib * TM * 16; i += THREADS) {
-            const int bits = load_agent(reinterpret_cast<const int *>(&s.sas[(size_t)mb * n_ib * (TM * 16) + i]));
-            s_sa[i / (TM * 16)][i % (TM * 16)] = __builtin_bit_cast(float, bits);
+        for (int i = tid; i < n_ib * TMD * 16; i += THREADS) {
+            const int ib = i / (TMD * 16), r = i - ib * (TMD * 16);
+            const int bits = load_agent(
+                reinterpret_cast<const int *>(&s.sas[(size_t)(mb * n_ib + ib) * (TM * 16) + part * (TMD * 16) + r]));
+            s_sa[ib][r] = __builtin_bit_cast(float, bits);
         }
         wait_vmcnt<0>();
         __syncthreads();
 
+        v4f accd[4][THD];
 #pragma unroll
         for (int a = 0; a < 4; a++)
 #pragma unroll
-            for (int t = 0; t < TH; t++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+            for (int t = 0; t < THD; t++) accd[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
         int cg = 0, cib = 0;
         // the ring's first two steps were issued above and have landed (wait_vmcnt<0>): from here on one younger step
         // stays in flight
@@ -460,20 +472,20 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
                     lds_barrier();
                     const int c0 = group_of(cg) << 6;
                     const float ws2 = s_w2s[(c0 >> 7) * n_ib + cib];
-                    mma_step<TH, AOPS>(a_ring + h * 8192, aq + cib * (TM * 2048) + g * (TH * 2048),
-                                       &s_sa[cib][g * (TH * 16) + n], ws2, ws2, acc, frag_lo, frag_hi,
-                                       [&](int i) { issue2_op((h + 2) % kStages, i); });
+                    mma_step<THD, AOPS>(a_ring + h * 8192, aq + cib * (TMD * 2048) + g * (THD * 2048),
+                                        &s_sa[cib][g * (THD * 16) + n], ws2, ws2, accd, frag_lo, frag_hi,
+                                        [&](int i) { issue2_op((h + 2) % kStages, i); });
                     advance2();
                     __builtin_amdgcn_sched_barrier(0);
                     cib++;
                     if (cib == n_ib) {
 #pragma unroll
-                        for (int t = 0; t < TH; t++) {
+                        for (int t = 0; t < THD; t++) {
                             if (valid[t] && cg < my_groups) {
                                 uint16_t *yp = s.y + (size_t)slot[t] * K + c0 + 16 * q;
 #pragma unroll
                                 for (int half = 0; half < 2; half++) {
-                                    const v4f lo = acc[2 * half][t] * tw[t], hi = acc[2 * half + 1][t] * tw[t];
+                                    const v4f lo = accd[2 * half][t] * tw[t], hi = accd[2 * half + 1][t] * tw[t];
                                     v4i o;
                                     o.x = (int)pack_bf16x2(lo[0], lo[1]);
                                     o.y = (int)pack_bf16x2(lo[2], lo[3]);
@@ -483,7 +495,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
                                 }
                             }
 #pragma unroll
-                            for (int a = 0; a < 4; a++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+                            for (int a = 0; a < 4; a++) accd[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
                         }
                         cib = 0;
                         cg++;
@@ -492,6 +504,19 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
             }
         }
         wait_vmcnt<0>();
+    };
+    // token parts of a DOWN item: the host picks the smallest divisor of TH whose tiles fit next to the weight ring
+    auto run_down = [&](int mb, int sub) {
+        const int cs = sub / s.nh, part = sub - cs * s.nh;
+        if (s.nh == 1) {
+            down_item(mb, cs, 0, std::integral_constant<int, TH>());
+        } else if (TH % 2 == 0 && s.nh == 2) {
+            down_item(mb, cs, part, std::integral_constant<int, (TH % 2 == 0 ? TH / 2 : TH)>());
+        } else if (TH % 3 == 0 && s.nh == 3) {
+            down_item(mb, cs, part, std::integral_constant<int, (TH % 3 == 0 ? TH / 3 : TH)>());
+        } else if (TH % 4 == 0 && s.nh == 4) {
+            down_item(mb, cs, part, std::integral_constant<int, (TH % 4 == 0 ? TH / 4 : TH)>());
+        }
     };
 
     // ---- item loop ------------------------------------------------------------------------------------------------
@@ -547,7 +572,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         if (up >= 0)
             up_item(qi * per_q + up / per_up, up % per_up);
         else
-            down_item(qi * per_q + down / per_down, down % per_down);
+            run_down(qi * per_q + down / per_down, down % per_down);
         __syncthreads();   // everybody is done with the item's LDS tables and rings before the next item refills them
     }
     if (tid == 0) {
@@ -619,7 +644,21 @@ int env_int(const char *name, int dflt)
     return e ? atoi(e) : dflt;
 }
 
-int tail_tiles(int n_ib) { return n_ib > kStages ? n_ib : kStages; }
+// Token parts of a DOWN item: the smallest divisor nh of th such that the requantised tiles of all n_ib slices of a
+// part (2 th / nh tiles per slice) fit next to the weight rings; 0 if none does.
+int token_parts(int th, int n_ib)
+{
+    for (int nh = 1; nh <= th; nh++)
+        if (th % nh == 0 && n_ib * (2 * th / nh) * 2048 <= kMaxTailBytes) return nh;
+    return 0;
+}
+
+// LDS behind the weight rings: the 3-stage ring of token tiles (UP items) or the requantised tiles of a part (DOWN)
+int tail_bytes(int th, int n_ib)
+{
+    const int up = kStages * 2 * th * 2048, down = n_ib * (2 * th / token_parts(th, n_ib)) * 2048;
+    return up > down ? up : down;
+}
 
 typedef void (*TileFn)(const TileParams);
 
@@ -653,7 +692,7 @@ bool tile_supported(int top_k, int M, int K, int N, int E, int sorted_num, int b
     const int tm = 2 * tiles_per_wave(block_m);
     const int n_ib = N / 256;
     const int64_t n_mb = ((int64_t)sorted_num + block_m - 1) / block_m;
-    return n_ib <= kTileMaxIb && tail_tiles(n_ib) * tm * 2048 <= kMaxTailBytes && K <= 128 * kTileMaxKb &&
+    return n_ib <= kTileMaxIb && token_parts(tm / 2, n_ib) > 0 && K <= 128 * kTileMaxKb &&
            (K / 128) * n_ib <= kTileMaxW2s && (int64_t)M * top_k <= kMaxSlots && n_mb * n_ib <= kMaxUnits;
 }
 
@@ -692,7 +731,8 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
     s.w_nt = env_int("ALPHA_MOE_TILE_NT", -1);
     if (s.lag < 1) s.lag = 1;
     const TileFn fn = pick(tm / 2);
-    const int lds_bytes = kARingBytes + tail_tiles(s.n_ib) * tm * 2048;
+    s.nh = token_parts(tm / 2, s.n_ib);
+    const int lds_bytes = kARingBytes + tail_bytes(tm / 2, s.n_ib);
     hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
                                          kARingBytes + kMaxTailBytes);
     if (err != hipSuccess) return err;
@@ -704,7 +744,7 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
             return 256;
         return n;
     }();
-    const int64_t items = (int64_t)s.n_mb_max * (s.n_ib + s.n_cs);
+    const int64_t items = (int64_t)s.n_mb_max * (s.n_ib + s.n_cs * s.nh);
     int grid = env_int("ALPHA_MOE_TILE_GRID", cus);
     if (grid > items) grid = (int)((items + 7) / 8 * 8);
     if (grid < 8) grid = 8;

@@ -81,10 +81,10 @@ def test_store_variant_overwrites_whatever_out_held(c1, knobs):
 
 
 def test_store_variant_fallback_kernel():
-    """Six 128-column slices with 128-row blocks exceed the tile kernel's LDS budget: the fallback kernel serves the call,
-    and its store variant overwrites too."""
+    """Nine 128-column slices are more than the tile kernel takes: the fallback kernel serves the call, and its store
+    variant overwrites too."""
     from alpha_moe_python.workloads import Shape
-    shape = Shape("fb", E=6, top_k=2, K=256, I=768, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0)
+    shape = Shape("fb", E=6, top_k=2, K=256, I=1152, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0)
     W = make_weights(shape, device=DEV, seed=5)
     P = make_problem(W, 150, seed=5)
     ref = oracle_out(P)
@@ -224,8 +224,8 @@ def q3_weights():
 
 @pytest.mark.parametrize("M,knobs", [(64, (16, 32, 8, 5)), (64, (32, 64, 4, 3)), (200, (64, 64, 4, 3)), (200, (128, 64, 4, 2))])
 def test_qwen3_30b_zipf_shard_against_oracle(q3_weights, M, knobs):
-    """Load imbalance: E=128, top_k=8, K=2048, I=768 (six 128-column slices), Zipf(1.2) expert popularity.  Row blocks
-    of 128 rows do not fit the tile kernel's LDS budget with six slices and take the fallback kernel."""
+    """Load imbalance: E=128, top_k=8, K=2048, I=768 (six 128-column slices), Zipf(1.2) expert popularity.  With six
+    slices a 128-row block's requantised tiles do not fit LDS at once: its DOWN items serve the tokens in two parts."""
     P = make_problem(q3_weights, M, seed=0)
     print(f"case q3 M={M} knobs {knobs}", flush=True)
     m = assert_parity(run_op(P, *knobs, via="c_abi"), oracle_out(P), f"q3 M={M} knobs {knobs}")
