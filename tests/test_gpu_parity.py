@@ -361,3 +361,36 @@ def test_hip_graph_capture_and_replay(c1, knobs, store):
         eager_problem = Problem(W, P.M, P2.x, P2.x_scale, P.topk_ids, P2.topk_weights)
         want = run_op(eager_problem, *knobs, via="c_abi")   # eager work between replays
         assert torch.equal(got, want), (knobs, store, rep)
+
+
+def test_random_small_shapes_and_knobs():
+    """Forty seeded random problems - token counts, expert counts, top_k, K (any multiple of 128, so also a single
+    64-column group pair and ragged column slabs), one to five 128-column slices, every row-block size of both kernels -
+    against the oracle."""
+    import random
+    from alpha_moe_python.workloads import Shape
+    rng = random.Random(20240607)
+    for case in range(40):
+        E = rng.choice([1, 2, 3, 5, 8, 17])
+        top_k = rng.randint(1, min(E, 4))
+        K = 128 * rng.choice([1, 2, 3, 5, 8, 9])
+        I = 128 * rng.choice([1, 1, 2, 3, 5])
+        M = rng.choice([1, 2, 7, 16, 33, 100, 257])
+        block_m = rng.choice([8, 16, 24, 32, 40, 64, 96, 128])
+        bn, wn = rng.choice([(64, 4), (32, 8)])
+        stages = rng.randint(1, 5)
+        shape = Shape(f"rnd{case}", E=E, top_k=top_k, K=K, I=I, shared_expert=False, routing="softmax_renorm",
+                      scaling_factor=rng.choice([1.0, 2.5]))
+        W = make_weights(shape, device=DEV, seed=case)
+        P = make_problem(W, M, seed=case)
+        print(f"case rnd{case} E={E} top_k={top_k} K={K} I={I} M={M} knobs {(block_m, bn, wn, stages)}", flush=True)
+        got = run_op(P, block_m, bn, wn, stages, via="c_abi")
+        # Tiny problems have few terms per output: where the device's and the oracle's fp32 sums of one intermediate
+        # value differ in the last bit and that value sits on an FP8 rounding boundary, it moves by a whole FP8 step
+        # (12.5 %), and an output element dominated by it by a few percent - seen as 1.2e-2 of the output range on one of
+        # these cases, identically from every kernel variant.  The bar here is therefore cosine >= 0.9999 and 2e-2 of
+        # the range (the reference's own test uses atol 2e-2, rtol 1e-1); the benchmark shapes keep the 1e-2 bar.
+        from oracle import moe_oracle as O
+        m = O.error_metrics(got, oracle_out(P))
+        assert torch.isfinite(got.float()).all()
+        assert m["cosine"] >= 0.9999 and m["max_abs_over_max_ref"] <= 2e-2 and m["allclose_2e-2_1e-1"], (case, m)
