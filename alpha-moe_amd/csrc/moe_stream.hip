@@ -303,20 +303,24 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         const int ksp = item - u * s.ks;
         const int mb = u / s.n_ib;
         const int ib = u - mb * s.n_ib;
+        // the rows' slot ids do not depend on the expert id: their loads go out before the wait for it (one memory
+        // round trip less at the head of every item)
+        const Routing<TM> r = load_routing<TM>(p, mb, n);
+        int row_id = -1;
+        if (tid < TM * 16) {
+            const int idx = mb * p.block_m + tid;
+            if (tid < p.block_m && idx < p.sorted_num) row_id = p.sorted_ids[idx];
+        }
         const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
         if (e < 0 || e >= p.E) return;
         const int kb0 = ksp * s.kbpi;
         const int nk = (s.nkb - kb0) < s.kbpi ? (s.nkb - kb0) : s.kbpi;
-        const Routing<TM> r = load_routing<TM>(p, mb, n);
 
         // per-item tables in LDS: token of every row, the unit's gate (row 2*ib) / up (row 2*ib+1) weight scales and
         // the tokens' activation scales over the item's K range
         if (tid < TM * 16) {
-            const int idx = mb * p.block_m + tid;
-            int id = -1;
-            if (tid < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
-            const int tk = id / p.top_k;
-            s_tok[tid] = (id >= 0 && tk < p.M) ? tk : 0;
+            const int tk = row_id / p.top_k;
+            s_tok[tid] = (row_id >= 0 && tk < p.M) ? tk : 0;
         }
         {
             const float *ws_rows = p.w_scale + ((size_t)e * (p.N >> 7) + 2 * ib) * s.nkb + kb0;
@@ -460,6 +464,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     auto down_item = [&](int item) {
         const int mb = item / s.n_cs;
         const int cs = item - mb * s.n_cs;
+        const Routing<TM> r = load_routing<TM>(p, mb, n);   // in flight together with the expert id
         const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
         if (e >= 0 && e < p.E) {
             const int n_ib = s.n_ib;
@@ -504,7 +509,6 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             const int nblk = (((t1 * 16) - 1) >> 7) - blk0 + 1;
             for (int i = tid; i < nblk * n_ib; i += THREADS)
                 s_sc[i] = p.w2_scale[((size_t)e * (K >> 7) + blk0) * n_ib + i];
-            const Routing<TM> r = load_routing<TM>(p, mb, n);
 
             if (tid == 0)
                 for (int ib = 0; ib < n_ib; ib++) spin_until_ge(&s.flag[mb * n_ib + ib], epoch, s.ctl);

@@ -146,7 +146,7 @@ def ds_weights():
 @pytest.mark.parametrize("M,knobs", [(1, (16, 32, 8, 5)), (4, (16, 64, 4, 4)), (16, (16, 64, 4, 3)), (64, (16, 32, 8, 3)),
                                      (64, (8, 64, 4, 2))])
 def test_deepseek_shard_decode_full_size(ds_weights, M, knobs):
-    """BASELINE decode configuration at its real size: E=257, top_k=9, K=7168, I=256."""
+    """The headline decode configuration at its real size: E=257, top_k=9, K=7168, I=256."""
     P = make_problem(ds_weights, M, seed=0)
     print(f"case ds M={M} knobs {knobs}", flush=True)
     m = assert_parity(run_op(P, *knobs), oracle_out(P), f"ds M={M} knobs {knobs}")
