@@ -138,6 +138,20 @@ __device__ __noinline__ void spin_until_ge(const int *addr, int target, StreamCt
     store_agent(&ctl->error, 1);
 }
 
+// The same for a whole wavefront and `count` <= 64 consecutive flags, one per lane: every poll is ONE load, so the wait
+// costs one round trip however many flags there are (a slice at a time it was I/128 dependent round trips).
+__device__ __noinline__ void spin_all_ge(const int *addr, int count, int target, StreamCtl *ctl)
+{
+    const int lane = threadIdx.x & 63;
+    for (int it = 0; it < (1 << 22); it++) {
+        const int v = lane < count ? load_agent(addr + lane) : target;
+        if (__all(v >= target)) return;
+        if (it < 16) __builtin_amdgcn_s_sleep(4);
+        else __builtin_amdgcn_s_sleep(32);
+    }
+    if (lane == 0) store_agent(&ctl->error, 1);
+}
+
 #ifdef ALPHA_MOE_TRACE
 // Debug builds only: per-item timestamps (100 MHz wall clock) for timeline analysis.
 __device__ unsigned long long g_trace[1 << 16][4];
@@ -465,6 +479,8 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         const int mb = item / s.n_cs;
         const int cs = item - mb * s.n_cs;
         const Routing<TM> r = load_routing<TM>(p, mb, n);   // in flight together with the expert id
+        // so is a first look at the flags of the block's slices (one lane each)
+        const int flag0 = (wave == 0 && lane < s.n_ib) ? load_agent(&s.flag[mb * s.n_ib + lane]) : epoch;
         const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
         if (e >= 0 && e < p.E) {
             const int n_ib = s.n_ib;
@@ -510,8 +526,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             for (int i = tid; i < nblk * n_ib; i += THREADS)
                 s_sc[i] = p.w2_scale[((size_t)e * (K >> 7) + blk0) * n_ib + i];
 
-            if (tid == 0)
-                for (int ib = 0; ib < n_ib; ib++) spin_until_ge(&s.flag[mb * n_ib + ib], epoch, s.ctl);
+            if (wave == 0 && !__all(flag0 >= epoch)) spin_all_ge(&s.flag[mb * n_ib], n_ib, epoch, s.ctl);
             __syncthreads();
             TRACE_MARK;
             if (wave == 0) prime();

@@ -172,15 +172,18 @@ __device__ __forceinline__ void store_agent(int *p, int v)
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Bounded wait of one thread for *addr >= target: ~4M polls a microsecond apart, then the sticky error flag.
-__device__ __noinline__ void tile_spin_until_ge(const int *addr, int target, StreamCtl *ctl)
+// Bounded wait of a wavefront for `count` <= 64 consecutive flags (one per lane) to reach `target`: one load per poll,
+// ~4M polls a microsecond apart, then the sticky error flag.
+__device__ __noinline__ void tile_spin_all_ge(const int *addr, int count, int target, StreamCtl *ctl)
 {
+    const int lane = threadIdx.x & 63;
     for (int it = 0; it < (1 << 22); it++) {
-        if (load_agent(addr) >= target) return;
+        const int v = lane < count ? load_agent(addr + lane) : target;
+        if (__all(v >= target)) return;
         if (it < 16) __builtin_amdgcn_s_sleep(4);
         else __builtin_amdgcn_s_sleep(32);
     }
-    store_agent(&ctl->error, 1);
+    if (lane == 0) store_agent(&ctl->error, 1);
 }
 
 // TH: 16-token tiles per wavefront; a row block has TM = 2 TH of them (block_m rounded up to 32 rows).
@@ -435,8 +438,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         // the weights do not depend on the up/gate phase: first two steps go out before the wait
         issue2(0);
         issue2(1);
-        if (tid == 0)
-            for (int ib = 0; ib < n_ib; ib++) tile_spin_until_ge(&s.flag[mb * n_ib + ib], epoch, s.ctl);
+        if (wave == 0) tile_spin_all_ge(&s.flag[mb * n_ib], n_ib, epoch, s.ctl);
         __syncthreads();
         // the requantised tiles of this part and their scales come from scratch into LDS: [slice][tile of the part]
         uint8_t *aq = xbuf;
