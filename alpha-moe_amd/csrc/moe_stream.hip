@@ -108,6 +108,13 @@ __device__ __forceinline__ void drain_vmem()
     __builtin_amdgcn_sched_barrier(0);
 }
 
+// Workgroup barrier that waits for this wavefront's LDS operations only: vector-memory operations stay in flight.
+__device__ __forceinline__ void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt()
 {
@@ -517,17 +524,18 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                     slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
                 }
             };
-            // Wavefront 0 polls the flags, and a poll returns behind everything the wavefront has in flight: it fills its
-            // ring after the poll, the others before.
-            if (wave != 0) prime();
-            // w2 scales of the 128-column blocks this item touches: s_sc[blk * n_ib + ib]
+            // w2 scales of the 128-column blocks this item touches: s_sc[blk * n_ib + ib].  Loaded BEFORE the ring is
+            // filled: waiting for them then leaves the ring's loads in flight.
             const int blk0 = (t0 * 16) >> 7;
             const int nblk = (((t1 * 16) - 1) >> 7) - blk0 + 1;
             for (int i = tid; i < nblk * n_ib; i += THREADS)
                 s_sc[i] = p.w2_scale[((size_t)e * (K >> 7) + blk0) * n_ib + i];
+            // Wavefront 0 polls the flags, and a poll returns behind everything the wavefront has in flight: it fills its
+            // ring after the poll, the others before.
+            if (wave != 0) prime();
 
             if (wave == 0 && !__all(flag0 >= epoch)) spin_all_ge(&s.flag[mb * n_ib], n_ib, epoch, s.ctl);
-            __syncthreads();
+            lds_barrier();   // the flags are up (and s_sc is written); the ring's loads stay in flight
             TRACE_MARK;
             if (wave == 0) prime();
 
