@@ -394,3 +394,25 @@ def test_random_small_shapes_and_knobs():
         m = O.error_metrics(got, oracle_out(P))
         assert torch.isfinite(got.float()).all()
         assert m["cosine"] >= 0.9999 and m["max_abs_over_max_ref"] <= 2e-2 and m["allclose_2e-2_1e-1"], (case, m)
+
+
+@pytest.mark.parametrize("knobs", [(16, 32, 8, 5), (64, 64, 4, 3)])
+def test_nothing_routed(c1, knobs):
+    """No live row block at all (num_tokens_post_padded = 0), and row blocks whose expert id is out of range: the adding
+    call leaves `out` as it was, the storing call writes zeros - both kernels."""
+    import alpha_moe
+    P, _ = c1
+    W = P.weights
+    block_m = knobs[0]
+    s_ids, e_ids, total = P.align(block_m)
+    for what in ("no blocks", "invalid experts"):
+        tot = torch.zeros_like(total) if what == "no blocks" else total
+        eid = e_ids if what == "no blocks" else torch.full_like(e_ids, -1)
+        for store in (False, True):
+            out = torch.full((P.M, P.shape.K), 0.5, dtype=torch.bfloat16, device=DEV)
+            op = torch.ops.alpha_moe.fused_moe_w8a8_up_down_store if store else torch.ops.alpha_moe.fused_moe_w8a8_up_down
+            print(f"case c1 {what} store={store} knobs {knobs}", flush=True)
+            op(P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, eid, tot, P.topk_weights, out, P.shape.top_k,
+               *knobs, P.shape.scaling_factor)
+            torch.cuda.synchronize()
+            assert torch.all(out == (0.0 if store else 0.5)), (what, store)
