@@ -29,7 +29,7 @@ sys.path.insert(0, ROOT)
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy of known size), for the
 # configurations that were profiled: profiles/moe_stream_kernel_ds_decode_M64_hbm_traffic.md
 #   profiles/moe_tile_kernel_ds_prefill_M8192_hbm_traffic.md (both kernels of a call)
-MEASURED_TRAFFIC_BYTES = {("ds", 64): 1295.3e6, ("ds", 8192): 4817.1e6}
+MEASURED_TRAFFIC_BYTES = {("ds", 64): 1294.9e6, ("ds", 8192): 4812.2e6}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
 DEFAULT_KNOBS = {"block_m": 16, "block_n": 32, "warp_n": 8, "stages": 5}
