@@ -38,6 +38,17 @@ def test_c_abi_workspace_is_reusable_without_clearing(c1):
     for bm, bn, wn, st in [(16, 64, 4, 2), (16, 64, 4, 2), (8, 32, 8, 3), (64, 64, 4, 2), (32, 32, 8, 1), (16, 64, 4, 4)]:
         print(f"case c1 shared workspace knobs {(bm, bn, wn, st)}", flush=True)
         assert_parity(run_op(P, bm, bn, wn, st, via="c_abi", workspace=ws), ref, f"shared ws {(bm, bn, wn, st)}")
+    # a second problem of another size on the same buffer, streaming and tile kernels taking turns
+    P2 = make_problem(P.weights, 150, seed=9)
+    need = max(alpha_moe.c_abi.alpha_moe_workspace_bytes(P2.shape.top_k, P2.M, P2.shape.K, P2.shape.N, P2.shape.E,
+                                                         P2.align(bm)[0].numel(), bm) for bm in (16, 64, 128))
+    ws2 = torch.zeros(max(need, ws.numel()), dtype=torch.uint8, device=DEV)
+    cases = [(P2, (128, 64, 4, 3)), (P, (16, 32, 8, 5)), (P2, (64, 64, 4, 3)), (P2, (16, 64, 4, 3)), (P, (96, 64, 4, 3))]
+    fresh = [run_op(prob, *knobs, via="c_abi") for prob, knobs in cases]   # each on a zero-filled buffer of its own
+    for rep in range(3):
+        for (prob, knobs), want in zip(cases, fresh):
+            print(f"case shared workspace round {rep} M={prob.M} knobs {knobs}", flush=True)
+            assert torch.equal(run_op(prob, *knobs, via="c_abi", workspace=ws2), want), (rep, prob.M, knobs)
 
 
 def test_c1_result_independent_of_every_knob(c1):
