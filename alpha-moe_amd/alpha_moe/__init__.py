@@ -31,6 +31,8 @@ c_abi.alpha_moe_fused_moe_w8a8_up_down.argtypes = (
     [ctypes.c_void_p] * 11 + [ctypes.c_int] * 10 + [ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p])
 c_abi.alpha_moe_fused_moe_w8a8_up_down_store.restype = ctypes.c_int
 c_abi.alpha_moe_fused_moe_w8a8_up_down_store.argtypes = c_abi.alpha_moe_fused_moe_w8a8_up_down.argtypes
+c_abi.alpha_moe_workspace_check.restype = ctypes.c_int
+c_abi.alpha_moe_workspace_check.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
 c_abi.alpha_moe_workspace_zero_bytes.restype = ctypes.c_size_t
 c_abi.alpha_moe_workspace_zero_bytes.argtypes = []
 c_abi.alpha_moe_workspace_bytes.restype = ctypes.c_size_t

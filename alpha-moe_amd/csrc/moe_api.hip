@@ -145,6 +145,18 @@ extern "C" int alpha_moe_fused_moe_w8a8_up_down_store(const uint8_t *x, const fl
                          warp_n, stages, scaling_factor, workspace, workspace_bytes, stream, 1);
 }
 
+extern "C" int alpha_moe_workspace_check(const void *workspace, void *stream)
+{
+    if (!workspace) return ALPHA_MOE_ERR_NULL_POINTER;
+    hipStream_t hs = static_cast<hipStream_t>(stream);
+    int flag = 0;
+    const StreamCtl *ctl = static_cast<const StreamCtl *>(workspace);
+    if (hipMemcpyAsync(&flag, &ctl->error, sizeof(int), hipMemcpyDeviceToHost, hs) != hipSuccess ||
+        hipStreamSynchronize(hs) != hipSuccess)
+        return ALPHA_MOE_ERR_LAUNCH;
+    return flag ? ALPHA_MOE_ERR_WAIT_EXPIRED : ALPHA_MOE_OK;
+}
+
 extern "C" size_t alpha_moe_workspace_zero_bytes(void) { return (stream_prefix_bytes() + 255) & ~(size_t)255; }
 
 extern "C" const char *alpha_moe_status_string(int status)
@@ -158,6 +170,9 @@ extern "C" const char *alpha_moe_status_string(int status)
     case ALPHA_MOE_ERR_STAGES: return "stages must be in [1, 5]";
     case ALPHA_MOE_ERR_WORKSPACE: return "workspace is null, not 256-byte aligned, or smaller than alpha_moe_workspace_bytes()";
     case ALPHA_MOE_ERR_LAUNCH: return "the HIP runtime refused the kernel launch";
+    case ALPHA_MOE_ERR_WAIT_EXPIRED:
+        return "a workgroup's bounded wait for another workgroup ran out in an earlier launch on this workspace: its "
+               "results are not valid (launches overlapping on one device, or a device that cannot hold the grid)";
     default: return "unknown status";
     }
 }

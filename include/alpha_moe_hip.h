@@ -23,7 +23,8 @@ enum alpha_moe_status {
     ALPHA_MOE_ERR_BLOCK_N_WARP_N = 4, /* (block_n, warp_n) not (64,4) or (32,8) */
     ALPHA_MOE_ERR_STAGES = 5,         /* stages not in 1..5 */
     ALPHA_MOE_ERR_LAUNCH = 6,         /* the HIP runtime refused the launch (see hipGetLastError) */
-    ALPHA_MOE_ERR_WORKSPACE = 7       /* workspace null, misaligned or smaller than alpha_moe_workspace_bytes() */
+    ALPHA_MOE_ERR_WORKSPACE = 7,      /* workspace null, misaligned or smaller than alpha_moe_workspace_bytes() */
+    ALPHA_MOE_ERR_WAIT_EXPIRED = 8    /* alpha_moe_workspace_check: a bounded wait between workgroups ran out */
 };
 
 /*
@@ -95,6 +96,15 @@ size_t alpha_moe_workspace_bytes(int top_k, int M, int K, int N, int num_experts
  * no scratch memory.
  */
 size_t alpha_moe_workspace_zero_bytes(void);
+
+/*
+ * Health of a workspace: waits for `stream`, then returns ALPHA_MOE_ERR_WAIT_EXPIRED if in any earlier launch on this
+ * workspace a workgroup gave up waiting for another (each such wait is bounded at a few seconds so that nothing
+ * hangs; the results of that launch are not valid), ALPHA_MOE_OK otherwise.  The flag is sticky until the prefix is
+ * zero-filled again.  Synchronises, so it is for tests and health checks, not for the serving loop.  The reference's
+ * kernel has no waits between thread blocks and no counterpart.
+ */
+int alpha_moe_workspace_check(const void *workspace, void *stream /* hipStream_t */);
 
 /*
  * The argument checks of the call above without touching the device: returns the status the launch would

@@ -91,6 +91,12 @@ def test_null_pointers_and_small_workspace_are_refused_without_touching_a_device
                                                       ctypes.c_void_p(4096), 1 << 40, None) == 3
 
 
+def test_workspace_check_refuses_a_null_workspace(lib):
+    lib.alpha_moe_workspace_check.restype = ctypes.c_int
+    lib.alpha_moe_workspace_check.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+    assert lib.alpha_moe_workspace_check(None, None) == 1
+
+
 def test_zeroed_prefix_is_small_and_inside_every_workspace(lib):
     lib.alpha_moe_workspace_zero_bytes.restype = ctypes.c_size_t
     lib.alpha_moe_workspace_zero_bytes.argtypes = []

@@ -427,3 +427,20 @@ def test_nothing_routed(c1, knobs):
                *knobs, P.shape.scaling_factor)
             torch.cuda.synchronize()
             assert torch.all(out == (0.0 if store else 0.5)), (what, store)
+
+
+def test_workspace_check_reports_an_expired_wait(c1):
+    """alpha_moe_workspace_check: 0 after ordinary launches of both kernels; 8 once the sticky word that a workgroup
+    writes when its bounded wait runs out is set (set here from the host: no kernel is made to wait)."""
+    import alpha_moe
+    P, ref = c1
+    need = max(alpha_moe.c_abi.alpha_moe_workspace_bytes(P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E,
+                                                         P.align(bm)[0].numel(), bm) for bm in (16, 64))
+    ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    for knobs in ((16, 32, 8, 5), (64, 64, 4, 3)):
+        assert_parity(run_op(P, *knobs, via="c_abi", workspace=ws), ref, f"knobs {knobs}")
+        assert alpha_moe.c_abi.alpha_moe_workspace_check(ws.data_ptr(), stream) == 0
+    ws.view(torch.int32)[3] = 1   # the control block's error word
+    rc = alpha_moe.c_abi.alpha_moe_workspace_check(ws.data_ptr(), stream)
+    assert rc == 8 and b"wait" in alpha_moe.c_abi.alpha_moe_status_string(rc)
