@@ -27,7 +27,9 @@
 // device holds at once (LDS granules included).  Another kernel occupying CUs only delays the items of the workgroups
 // it keeps out; two launches of THIS kernel that share a device at the same time could keep each other's workgroups
 // out for good, so launches on one device are serialised by the caller (one stream, or one workspace - which
-// concurrent launches may not share anyway).  Each spin is bounded and sets ctl->error instead of hanging.  The workspace starts zero-filled; its first kPrefixBytes hold the control block,
+// concurrent launches may not share anyway), or the caller sets ALPHA_MOE_STRICT_QUEUE=1: then the first item comes
+// from the counter as well, only running workgroups ever hold items, and the queue drains with any number of them
+// resident (a microsecond or two slower at decode sizes).  Each spin is bounded and sets ctl->error instead of hanging.  The workspace starts zero-filled; its first kPrefixBytes hold the control block,
 // the arrival counters (reset by the last arrival) and epoch-stamped flags, so nothing has to be cleared between
 // launches; the rest (aq, sa, hpart, y) is only ever read after it was written in the same launch.
 //
@@ -70,6 +72,7 @@ struct StreamPlan {
     int n_fc;        // FIN items per token
     int lag;         // row blocks between a block's UP items and its DOWN items in the queue
     int bm_pad;
+    int strict_queue;   // every item, the first one too, comes from the counter: correct with any number of resident workgroups
 };
 
 typedef const void __attribute__((address_space(1))) * gptr_t;
@@ -274,7 +277,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     auto fetch_next = [&]() {
         // the first gridDim.x items are handed out by workgroup index, the counter hands out the rest
         if (tid == 0 && next_item < 0)
-            next_item = (int)gridDim.x +
+            next_item = (s.strict_queue ? 0 : (int)gridDim.x) +
                         __hip_atomic_fetch_add(&s.ctl->head, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
 
@@ -672,6 +675,13 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         return 2;
     };
     int item = blockIdx.x;   // no round trip to the queue before the first item
+    if (s.strict_queue) {    // unless the caller cannot promise that the whole grid is resident at once
+        fetch_next();
+        if (tid == 0) s_bcast[0] = next_item;
+        __syncthreads();
+        item = __builtin_amdgcn_readfirstlane(s_bcast[0]);
+        __syncthreads();
+    }
     while (item < total) {
         TRACE_BEGIN;
         next_item = -1;
@@ -935,6 +945,7 @@ hipError_t launch_stream(const MoeParams &p, int warp_n, int stages, void *works
     s.n_cs = h.n_cs;
     s.n_fc = h.n_fc;
     s.lag = h.lag;
+    s.strict_queue = env_int("ALPHA_MOE_STRICT_QUEUE", 0) != 0;
 
     const Variant v = pick((p.block_m + 15) / 16, warp_n, stages);
     const int lds_bytes = v.ring_bytes + h.n_ib * v.tm * 2048;

@@ -444,3 +444,22 @@ def test_workspace_check_reports_an_expired_wait(c1):
     ws.view(torch.int32)[3] = 1   # the control block's error word
     rc = alpha_moe.c_abi.alpha_moe_workspace_check(ws.data_ptr(), stream)
     assert rc == 8 and b"wait" in alpha_moe.c_abi.alpha_moe_status_string(rc)
+
+
+def test_strict_queue_survives_a_grid_the_device_cannot_hold(ds_weights, monkeypatch):
+    """With ALPHA_MOE_STRICT_QUEUE=1 no workgroup owns an item before it runs, so even a grid of four times what the
+    device holds at once (workgroups that start only when others have left) finishes at once and correctly - the
+    property callers need who overlap launches on several streams.  The default mode refuses nothing but would stall
+    here, which is why the host never asks for such a grid."""
+    import time
+    P = make_problem(ds_weights, 16, seed=4)
+    base = run_op(P, 16, 32, 8, 5, via="c_abi")
+    monkeypatch.setenv("ALPHA_MOE_STRICT_QUEUE", "1")
+    assert torch.equal(run_op(P, 16, 32, 8, 5, via="c_abi"), base)
+    monkeypatch.setenv("ALPHA_MOE_GRID", "1024")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    got = run_op(P, 16, 32, 8, 5, via="c_abi")
+    dt = time.perf_counter() - t0
+    assert dt < 0.5, f"launch took {dt:.2f} s"
+    assert torch.equal(got, base)
