@@ -463,3 +463,41 @@ def test_strict_queue_survives_a_grid_the_device_cannot_hold(ds_weights, monkeyp
     dt = time.perf_counter() - t0
     assert dt < 0.5, f"launch took {dt:.2f} s"
     assert torch.equal(got, base)
+
+
+def test_strict_queue_two_streams_at_once(ds_weights, monkeypatch):
+    """Two launches in flight at the same time on two streams, each with a workspace of its own, in the mode made for
+    it: both finish at once and agree bit for bit with launches that ran alone."""
+    import time
+    import alpha_moe
+    monkeypatch.setenv("ALPHA_MOE_STRICT_QUEUE", "1")
+    P1 = make_problem(ds_weights, 32, seed=5)
+    P2 = make_problem(ds_weights, 24, seed=6)
+    knobs = (16, 32, 8, 5)
+    alone = [run_op(P, *knobs, via="c_abi") for P in (P1, P2)]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs, keep = [], []
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for rep in range(5):
+        for P, st in zip((P1, P2), streams):
+            with torch.cuda.stream(st):
+                s_ids, e_ids, total = P.align(knobs[0])
+                need = alpha_moe.c_abi.alpha_moe_workspace_bytes(P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E,
+                                                                 s_ids.numel(), knobs[0])
+                ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+                out = torch.zeros((P.M, P.shape.K), dtype=torch.bfloat16, device=DEV)
+                W = P.weights
+                rc = alpha_moe.c_abi.alpha_moe_fused_moe_w8a8_up_down(
+                    P.x.data_ptr(), P.x_scale.data_ptr(), W.w1.data_ptr(), W.w1_scale.data_ptr(), W.w2.data_ptr(),
+                    W.w2_scale.data_ptr(), out.data_ptr(), s_ids.data_ptr(), e_ids.data_ptr(), total.data_ptr(),
+                    P.topk_weights.data_ptr(), P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E, s_ids.numel(),
+                    *knobs, float(P.shape.scaling_factor), ws.data_ptr(), ws.numel(), st.cuda_stream)
+                assert rc == 0
+                outs.append(out)
+                keep.append((ws, s_ids, e_ids, total))
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert dt < 1.0, f"ten overlapping launches took {dt:.2f} s"
+    for i, out in enumerate(outs):
+        assert torch.equal(out, alone[i % 2]), i
