@@ -75,93 +75,6 @@ struct StreamPlan {
     int strict_queue;   // every item, the first one too, comes from the counter: correct with any number of resident workgroups
 };
 
-typedef const void __attribute__((address_space(1))) * gptr_t;
-typedef void __attribute__((address_space(3))) * lptr_t;
-
-// 64 lanes x 16 bytes, memory -> LDS at lds + lane*16, bypassing VGPRs.  AUX: 0 default, 2 non-temporal, 16 agent scope
-template <int AUX>
-__device__ __forceinline__ void dma16(const uint8_t *g, uint8_t *lds)
-{
-    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uint32_t)(uintptr_t)lds, 16, 0, AUX);
-}
-
-// Agent-scope (sc1) accesses for data that crosses workgroups inside one launch.  The loads are invisible to the
-// compiler's wait-count insertion: drain_vmem() before using their results.
-__device__ __forceinline__ v4i ldg128_agent(const void *p)
-{
-    v4i r;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(r) : "v"(p) : "memory");
-    return r;
-}
-__device__ __forceinline__ void stg32_agent(void *p, uint32_t v)
-{
-    asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-}
-__device__ __forceinline__ void stg128_agent(void *p, v4f v)
-{
-    // The hardware reads the data registers of a store wider than 64 bits a few cycles after issue; the compiler's
-    // hazard recognizer cannot see into inline asm, so the wait states before those registers may be overwritten
-    // are spelled out here.
-    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" ::"v"(p), "v"(v) : "memory");
-}
-// all of this wavefront's vector-memory operations (loads, stores, direct-to-LDS loads) have completed
-__device__ __forceinline__ void drain_vmem()
-{
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-}
-
-// Workgroup barrier that waits for this wavefront's LDS operations only: vector-memory operations stay in flight.
-__device__ __forceinline__ void lds_barrier()
-{
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt()
-{
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-    __builtin_amdgcn_sched_barrier(0);   // nothing that consumes the awaited data may be scheduled above the wait
-}
-
-__device__ __forceinline__ int load_agent(const int *p)
-{
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void store_agent(int *p, int v)
-{
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Bounded wait for *addr >= target (one thread).  ~4M polls with a sleep between them, i.e. seconds.  The sleep grows
-// from 0.1 us to 0.9 us: a hundred workgroups polling one address every 0.2 us keep that L2 channel busy enough to
-// slow the loads of the workgroups still streaming weights threefold (measured).
-__device__ __noinline__ void spin_until_ge(const int *addr, int target, StreamCtl *ctl)
-{
-    for (int it = 0; it < (1 << 22); it++) {
-        if (load_agent(addr) >= target) return;
-        if (it < 16) __builtin_amdgcn_s_sleep(4);
-        else __builtin_amdgcn_s_sleep(32);
-    }
-    store_agent(&ctl->error, 1);
-}
-
-// The same for a whole wavefront and `count` <= 64 consecutive flags, one per lane: every poll is ONE load, so the wait
-// costs one round trip however many flags there are (a slice at a time it was I/128 dependent round trips).
-__device__ __noinline__ void spin_all_ge(const int *addr, int count, int target, StreamCtl *ctl)
-{
-    const int lane = threadIdx.x & 63;
-    for (int it = 0; it < (1 << 22); it++) {
-        const int v = lane < count ? load_agent(addr + lane) : target;
-        if (__all(v >= target)) return;
-        if (it < 16) __builtin_amdgcn_s_sleep(4);
-        else __builtin_amdgcn_s_sleep(32);
-    }
-    if (lane == 0) store_agent(&ctl->error, 1);
-}
-
 #ifdef ALPHA_MOE_TRACE
 // Debug builds only: per-item timestamps (100 MHz wall clock) for timeline analysis.
 __device__ unsigned long long g_trace[1 << 16][4];

@@ -64,41 +64,6 @@ struct TileParams {
     int w_nt;         // weights with non-temporal loads: 1 always, 0 never, -1 for experts with a single row block
 };
 
-typedef const void __attribute__((address_space(1))) * gptr_t;
-typedef void __attribute__((address_space(3))) * lptr_t;
-
-// memory -> LDS without passing VGPRs: lane l's 16 (4) bytes land at lds + 16 l (4 l); the global address is per lane
-__device__ __forceinline__ void dma16(const void *g, void *lds)
-{
-    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uintptr_t)lds, 16, 0, 0);
-}
-// the same, non-temporal: for weight streams that nobody else reads soon (see the streaming kernel's header for the rates)
-__device__ __forceinline__ void dma16_nt(const void *g, void *lds)
-{
-    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uintptr_t)lds, 16, 0, 2);
-}
-__device__ __forceinline__ void dma4(const void *g, void *lds)
-{
-    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uintptr_t)lds, 4, 0, 0);
-}
-
-// The compiler does not count direct-to-LDS loads; the loops below do.
-template <int N>
-__device__ __forceinline__ void wait_vmcnt()
-{
-    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
-    __builtin_amdgcn_sched_barrier(0);
-}
-
-// Workgroup barrier that waits for this wavefront's LDS operations only (__syncthreads would also drain every
-// outstanding global load, and with them the prefetches in flight).
-__device__ __forceinline__ void lds_barrier()
-{
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    __builtin_amdgcn_sched_barrier(0);
-}
-
 // One step of a wavefront: 4 weight tiles x TH token tiles, all from LDS.  acc[k][t] += (A_k x B_t) * row[t] * sc[k & 1]
 // with row[] a per-token factor in LDS (16 floats per tile, already offset to this lane's token).  The product of
 // (k, t) is scaled into its accumulator behind the matrix instruction of (k, t + 1).
@@ -151,39 +116,6 @@ __device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *
     }
 #pragma unroll
     for (int k = 0; k < 4; k++) acc[k][TH - 1] += prev[k] * ((k & 1) ? p1 : p0);
-}
-
-// Agent-scope accesses for what crosses workgroups (and XCDs, whose L2s are not coherent with each other) inside the
-// launch: requantised tiles, their scales, the flags.
-__device__ __forceinline__ void stg32_agent(void *p, uint32_t v)
-{
-    asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-}
-__device__ __forceinline__ void dma16_agent(const void *g, void *lds)
-{
-    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uintptr_t)lds, 16, 0, 16);   // sc1
-}
-__device__ __forceinline__ int load_agent(const int *p)
-{
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void store_agent(int *p, int v)
-{
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// Bounded wait of a wavefront for `count` <= 64 consecutive flags (one per lane) to reach `target`: one load per poll,
-// ~4M polls a microsecond apart, then the sticky error flag.
-__device__ __noinline__ void tile_spin_all_ge(const int *addr, int count, int target, StreamCtl *ctl)
-{
-    const int lane = threadIdx.x & 63;
-    for (int it = 0; it < (1 << 22); it++) {
-        const int v = lane < count ? load_agent(addr + lane) : target;
-        if (__all(v >= target)) return;
-        if (it < 16) __builtin_amdgcn_s_sleep(4);
-        else __builtin_amdgcn_s_sleep(32);
-    }
-    if (lane == 0) store_agent(&ctl->error, 1);
 }
 
 // TH: 16-token tiles per wavefront; a row block has TM = 2 TH of them (block_m rounded up to 32 rows).
@@ -289,12 +221,12 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
                 const int up = i >> 1, h = i & 1;
                 const uint8_t *src = wbase + (size_t)(h * 16 + 8 * up) * K + (size_t)kc * 128 + ld_chunk[h];
                 uint8_t *dst = a_ring + stage * 8192 + (2 * g + up) * 2048 + h * 1024;
-                if (nt) dma16_nt(src, dst);
-                else dma16(src, dst);
+                if (nt) dma16<2>(src, dst);
+                else dma16<0>(src, dst);
             } else if (i < AOPS + 2) {
                 const int part = i - AOPS;
                 uint8_t *dst = x_real ? xbuf + stage * (TM * 2048) + wave * 2048 : s_dummy;
-                dma16(gx[part] + (size_t)kc * 128, dst + part * 1024);
+                dma16<0>(gx[part] + (size_t)kc * 128, dst + part * 1024);
             } else {
                 float *sdst = x_real ? &s_xs[stage][wave * 16] : reinterpret_cast<float *>(s_dummy + 2048);
                 if (lane < 16) dma4(gxs + kc, sdst);
@@ -420,8 +352,8 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
             const int k = 2 * g + (i >> 1), h = i & 1;
             const uint8_t *src = w2base + (size_t)(c0 + 32 * h + 4 * k) * I + lib * 128 + ld_chunk[h];
             uint8_t *dst = a_ring + stage * 8192 + k * 2048 + h * 1024;
-            if (nt) dma16_nt(src, dst);
-            else dma16(src, dst);
+            if (nt) dma16<2>(src, dst);
+            else dma16<0>(src, dst);
         };
         auto advance2 = [&]() {
             lib++;
@@ -438,15 +370,15 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         // the weights do not depend on the up/gate phase: first two steps go out before the wait
         issue2(0);
         issue2(1);
-        if (wave == 0) tile_spin_all_ge(&s.flag[mb * n_ib], n_ib, epoch, s.ctl);
+        if (wave == 0) spin_all_ge(&s.flag[mb * n_ib], n_ib, epoch, s.ctl);
         __syncthreads();
         // the requantised tiles of this part and their scales come from scratch into LDS: [slice][tile of the part]
         uint8_t *aq = xbuf;
         for (int i = wave; i < n_ib * TMD; i += 8) {
             const int ib = i / TMD, tt = i - ib * TMD;
             const uint8_t *src = s.aqs + ((size_t)(mb * n_ib + ib) * TM + part * TMD + tt) * 2048 + lane * 16;
-            dma16_agent(src, aq + i * 2048);
-            dma16_agent(src + 1024, aq + i * 2048 + 1024);
+            dma16<16>(src, aq + i * 2048);
+            dma16<16>(src + 1024, aq + i * 2048 + 1024);
         }
         for (int i = tid; i < n_ib * TMD * 16; i += THREADS) {
             const int ib = i / (TMD * 16), r = i - ib * (TMD * 16);
