@@ -37,3 +37,18 @@ def test_cpu_tensors_are_refused():
             torch.ones((E, K // 128, N // 256)), torch.zeros(M * top_k + E * 15, dtype=torch.int32),
             torch.zeros(10, dtype=torch.int32), torch.zeros(1, dtype=torch.int32), torch.ones((M, top_k)),
             torch.zeros((M, K), dtype=torch.bfloat16), top_k, 16, 64, 4, 3, 1.0)
+
+
+def test_store_variant_has_the_same_schema_and_a_fake_impl():
+    a = str(torch.ops.alpha_moe.fused_moe_w8a8_up_down.default._schema)
+    b = str(torch.ops.alpha_moe.fused_moe_w8a8_up_down_store.default._schema)
+    assert b == a.replace("fused_moe_w8a8_up_down(", "fused_moe_w8a8_up_down_store(")
+    M, K, N, E, top_k = 4, 256, 256, 3, 2
+    meta = lambda shape, dt: torch.empty(shape, dtype=dt, device="meta")
+    out = meta((M, K), torch.bfloat16)
+    res = alpha_moe_ops.fused_moe_w8a8_up_down_store(
+        meta((M, K), torch.float8_e4m3fn), meta((M, K // 128), torch.float32), meta((E, N, K), torch.float8_e4m3fn),
+        meta((E, N // 128, K // 128), torch.float32), meta((E, K, N // 2), torch.float8_e4m3fn),
+        meta((E, K // 128, N // 256), torch.float32), meta((M * top_k + E * 15,), torch.int32), meta((10,), torch.int32),
+        meta((1,), torch.int32), meta((M, top_k), torch.float32), out, top_k, 16, 64, 4, 3, 1.0)
+    assert res is out
