@@ -31,6 +31,8 @@ c_abi.alpha_moe_fused_moe_w8a8_up_down.argtypes = (
     [ctypes.c_void_p] * 11 + [ctypes.c_int] * 10 + [ctypes.c_float, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p])
 c_abi.alpha_moe_fused_moe_w8a8_up_down_store.restype = ctypes.c_int
 c_abi.alpha_moe_fused_moe_w8a8_up_down_store.argtypes = c_abi.alpha_moe_fused_moe_w8a8_up_down.argtypes
+c_abi.alpha_moe_set_tunable.restype = ctypes.c_int
+c_abi.alpha_moe_set_tunable.argtypes = [ctypes.c_char_p, ctypes.c_int, ctypes.c_int]
 c_abi.alpha_moe_workspace_check.restype = ctypes.c_int
 c_abi.alpha_moe_workspace_check.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
 c_abi.alpha_moe_workspace_zero_bytes.restype = ctypes.c_size_t
@@ -49,3 +51,10 @@ c_abi.alpha_moe_moe_align_block_size.argtypes = (
                                               ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p])
 
 __version__ = c_abi.alpha_moe_version().decode()
+
+
+def set_tunable(name: str, value=None) -> None:
+    """Install (``value`` an int) or clear (``None``) one of the library's tuning overrides (experiments and tests)."""
+    rc = c_abi.alpha_moe_set_tunable(name.encode(), 0 if value is None else int(value), 0 if value is None else 1)
+    if rc != 0:
+        raise ValueError(f"unknown tunable {name!r}")

@@ -2,24 +2,41 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "moe_common.hpp"
 
 using namespace alpha_moe;
 
 namespace {
 
-// ALPHA_MOE_PATH=direct|stream|tile forces one kernel family where it applies (for experiments).
-int forced_path()
+// Tuning overrides: name (also the environment variable read once at first use), current value.
+struct TunableSlot {
+    const char *name;
+    int value;
+};
+TunableSlot g_tunables[kTunCount] = {
+    {"ALPHA_MOE_PATH", kTunableUnset},        {"ALPHA_MOE_STRICT_QUEUE", kTunableUnset},
+    {"ALPHA_MOE_KBPI", kTunableUnset},        {"ALPHA_MOE_TPI", kTunableUnset},
+    {"ALPHA_MOE_LAG", kTunableUnset},         {"ALPHA_MOE_GRID", kTunableUnset},
+    {"ALPHA_MOE_TILE_GPS", kTunableUnset},    {"ALPHA_MOE_TILE_LAG", kTunableUnset},
+    {"ALPHA_MOE_TILE_GRID", kTunableUnset},   {"ALPHA_MOE_TILE_NT", kTunableUnset},
+};
+
+void load_tunables_once()
 {
-    static const int v = [] {
-        const char *e = getenv("ALPHA_MOE_PATH");
-        if (!e) return 0;
-        if (!strcmp(e, "direct")) return 1;
-        if (!strcmp(e, "stream")) return 2;
-        if (!strcmp(e, "tile")) return 3;
-        return 0;
+    static const bool done = [] {
+        for (TunableSlot &t : g_tunables) {
+            const char *e = getenv(t.name);
+            if (!e) continue;
+            if (!strcmp(t.name, "ALPHA_MOE_PATH"))
+                t.value = !strcmp(e, "direct") ? 1 : !strcmp(e, "stream") ? 2 : !strcmp(e, "tile") ? 3 : kTunableUnset;
+            else
+                t.value = atoi(e);
+        }
+        return true;
     }();
-    return v;
+    (void)done;
 }
 
 enum Path { kDirect, kStream, kTile };
@@ -30,7 +47,7 @@ Path choose_path(int top_k, int M, int K, int N, int E, int sorted_num, int bloc
 {
     const bool s_ok = stream_supported(top_k, M, K, N, E, sorted_num, block_m);
     const bool t_ok = tile_supported(top_k, M, K, N, E, sorted_num, block_m);
-    const int f = forced_path();
+    const int f = tunable(kTunPath, 0);
     if (f == 1) return kDirect;
     if (f == 2 && s_ok) return kStream;
     if (f == 3 && t_ok) return kTile;
@@ -40,6 +57,25 @@ Path choose_path(int top_k, int M, int K, int N, int E, int sorted_num, int bloc
 }
 
 }  // namespace
+
+int alpha_moe::tunable(Tunable which, int dflt)
+{
+    load_tunables_once();
+    const int v = g_tunables[which].value;
+    return v == kTunableUnset ? dflt : v;
+}
+
+extern "C" int alpha_moe_set_tunable(const char *name, int value, int set)
+{
+    if (!name) return ALPHA_MOE_ERR_NULL_POINTER;
+    load_tunables_once();
+    for (TunableSlot &t : g_tunables)
+        if (!strcmp(t.name, name)) {
+            t.value = set ? value : kTunableUnset;
+            return ALPHA_MOE_OK;
+        }
+    return ALPHA_MOE_ERR_SHAPE;
+}
 
 extern "C" int alpha_moe_validate(int top_k, int M, int K, int N, int num_experts, int sorted_num, int block_m,
                                   int block_n, int warp_n, int stages)
@@ -177,4 +213,4 @@ extern "C" const char *alpha_moe_status_string(int status)
     }
 }
 
-extern "C" const char *alpha_moe_version(void) { return "0.2"; }
+extern "C" const char *alpha_moe_version(void) { return "0.3"; }

@@ -124,6 +124,13 @@ __device__ __forceinline__ void wait_vmcnt()
 // all of this wavefront's vector-memory operations (loads, stores, direct-to-LDS loads) have completed
 __device__ __forceinline__ void drain_vmem() { wait_vmcnt<0>(); }
 
+// all of this wavefront's LDS operations (reads into registers included) have completed
+__device__ __forceinline__ void wait_lds_reads()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 // Workgroup barrier that waits for this wavefront's LDS operations only (__syncthreads would also drain every
 // outstanding global load, and with them the prefetches in flight).
 __device__ __forceinline__ void lds_barrier()
@@ -133,13 +140,25 @@ __device__ __forceinline__ void lds_barrier()
 }
 
 // Agent-scope (sc1) accesses for data that crosses workgroups - and XCDs, whose L2s are not coherent with each other -
-// inside one launch.  The asm ones are invisible to the compiler's wait-count insertion: drain_vmem() before using
-// what they load, or before telling anybody about what they stored.
+// inside one launch.  The asm ones are invisible to the compiler's wait-count insertion: drain_vmem_into() the
+// registers they load before using them, drain_vmem() before telling anybody about what they stored.
 __device__ __forceinline__ v4i ldg128_agent(const void *p)
 {
     v4i r;
     asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(r) : "v"(p) : "memory");
     return r;
+}
+// Wait for everything this wavefront has in flight and hand the registers of up to eight ldg128_agent() loads over
+// to the compiler only now: as in/out operands of the wait they cannot be read - and their registers cannot be given
+// to anything else - before the data has landed.  (A bare wait would not do: the compiler sees an asm load's result as
+// ready at once, and a late-landing load then overwrites whatever it moved into those registers, addresses included.)
+__device__ __forceinline__ void drain_vmem_into(v4i (&r)[8])
+{
+    asm volatile("s_waitcnt vmcnt(0)"
+                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7])
+                 :
+                 : "memory");
+    __builtin_amdgcn_sched_barrier(0);
 }
 __device__ __forceinline__ void stg32_agent(void *p, uint32_t v)
 {
@@ -163,8 +182,9 @@ __device__ __forceinline__ void store_agent(int *p, int v)
 
 // ---- workspace prefix shared by the kernel families --------------------------------------------------------
 // The first kPrefixBytes of the workspace are zero-initialised by the caller once and maintained by the kernels:
-// counters return to zero by themselves, flags are stamped with a launch epoch that only ever grows.  Its size
-// does not depend on the problem, so calls of different sizes can share one buffer.
+// counters return to zero by themselves, flags are stamped with a launch epoch that grows by one per launch and is
+// compared modulo 2^32 (reached()), so it may wrap.  Its size does not depend on the problem, so calls of different
+// sizes can share one buffer.
 constexpr int kMaxUnits = 1 << 16;   // most (row block, slice) units of one streaming launch
 constexpr int kMaxSlots = 1 << 18;   // most (token, slot) rows whose results go through per-slot rows
 
@@ -194,10 +214,13 @@ constexpr size_t kPrefixBytes = kOffLive + sizeof(int) * kMaxSlots;
 // every 0.2 us keep that L2 channel busy enough to slow the loads of the workgroups still streaming weights threefold
 // (measured).
 // One thread, one address:
+// "a >= b" for counters and epochs that wrap around: true while a is at most 2^31 - 1 steps ahead of b
+__device__ __forceinline__ bool reached(int a, int b) { return (int)((unsigned)a - (unsigned)b) >= 0; }
+
 __device__ __noinline__ inline void spin_until_ge(const int *addr, int target, StreamCtl *ctl)
 {
     for (int it = 0; it < (1 << 22); it++) {
-        if (load_agent(addr) >= target) return;
+        if (reached(load_agent(addr), target)) return;
         if (it < 16) __builtin_amdgcn_s_sleep(4);
         else __builtin_amdgcn_s_sleep(32);
     }
@@ -210,12 +233,31 @@ __device__ __noinline__ inline void spin_all_ge(const int *addr, int count, int 
     const int lane = threadIdx.x & 63;
     for (int it = 0; it < (1 << 22); it++) {
         const int v = lane < count ? load_agent(addr + lane) : target;
-        if (__all(v >= target)) return;
+        if (__all(reached(v, target))) return;
         if (it < 16) __builtin_amdgcn_s_sleep(4);
         else __builtin_amdgcn_s_sleep(32);
     }
     if (lane == 0) store_agent(&ctl->error, 1);
 }
+
+// ---- tuning overrides (experiments and tests) ---------------------------------------------------------------
+// Read from the environment ONCE, when the library is first used, and changed afterwards only through
+// alpha_moe_set_tunable(): no launch ever calls getenv.  A value of kTunableUnset means "the library decides".
+constexpr int kTunableUnset = INT32_MIN;
+enum Tunable {
+    kTunPath,          // ALPHA_MOE_PATH: 1 direct, 2 stream, 3 tile (where the family applies)
+    kTunStrictQueue,   // ALPHA_MOE_STRICT_QUEUE: 0 hands the first gridDim.x items of the streaming kernel out by index
+    kTunKbpi,          // ALPHA_MOE_KBPI: K blocks per UP item of the streaming kernel
+    kTunTpi,           // ALPHA_MOE_TPI: 16-column tiles per DOWN item of the streaming kernel
+    kTunLag,           // ALPHA_MOE_LAG: row blocks between a block's UP and DOWN items in the streaming queue
+    kTunGrid,          // ALPHA_MOE_GRID: workgroups of the streaming kernel
+    kTunTileGps,       // ALPHA_MOE_TILE_GPS: 64-column groups per DOWN item of the tile kernel
+    kTunTileLag,       // ALPHA_MOE_TILE_LAG
+    kTunTileGrid,      // ALPHA_MOE_TILE_GRID
+    kTunTileNt,        // ALPHA_MOE_TILE_NT: non-temporal weight loads 1 always, 0 never
+    kTunCount
+};
+int tunable(Tunable which, int dflt);   // the override if one is set, else dflt
 
 // ---- host-side launchers, one per kernel family (each in its own translation unit) -------------------------
 

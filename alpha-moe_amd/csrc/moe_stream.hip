@@ -20,18 +20,16 @@
 //
 // There is no floating-point atomic anywhere: the result is bit-reproducible from run to run.
 //
-// Every wait is on items EARLIER in the queue, and items never wait on later ones.  The first gridDim.x items belong to
-// the workgroups by index (no round trip to the counter, no storm of same-address atomics at the start), the rest
-// go to whoever asks the counter next.  The queue therefore drains as long as every workgroup of the grid becomes
-// resident without one of this launch's workgroups having to retire first: the host sizes the grid to what the
-// device holds at once (LDS granules included).  Another kernel occupying CUs only delays the items of the workgroups
-// it keeps out; two launches of THIS kernel that share a device at the same time could keep each other's workgroups
-// out for good, so launches on one device are serialised by the caller (one stream, or one workspace - which
-// concurrent launches may not share anyway), or the caller sets ALPHA_MOE_STRICT_QUEUE=1: then the first item comes
-// from the counter as well, only running workgroups ever hold items, and the queue drains with any number of them
-// resident (a microsecond or two slower at decode sizes).  Each spin is bounded and sets ctl->error instead of hanging.  The workspace starts zero-filled; its first kPrefixBytes hold the control block,
-// the arrival counters (reset by the last arrival) and epoch-stamped flags, so nothing has to be cleared between
-// launches; the rest (aq, sa, hpart, y) is only ever read after it was written in the same launch.
+// Every wait is on items EARLIER in the queue, and items never wait on later ones.  Every item, the first one of a
+// workgroup too, comes from one counter: only running workgroups ever hold items, so the queue drains with any number
+// of workgroups resident - launches may overlap on a device (several streams, other persistent kernels) without
+// being able to starve each other.  (ALPHA_MOE_STRICT_QUEUE=0 hands the first gridDim.x items out by workgroup index
+// instead, which saves the first round trip to the counter but is only correct when the whole grid is resident at
+// once; it is an experiment switch, not a mode to serve with.)  Each spin is bounded and sets ctl->error instead of
+// hanging; the items that write `out` then fill it with NaN, in that launch and in every later one on the workspace.
+// The workspace starts zero-filled; its first kPrefixBytes hold the control block, the arrival counters (reset by the
+// last arrival) and epoch-stamped flags, so nothing has to be cleared between launches; the rest (aq, sa, hpart, y)
+// is only ever read after it was written in the same launch.
 //
 // Data movement: weights go HBM -> LDS with non-temporal global_load_lds_dwordx4 (measured on MI355X: 6.9 TB/s
 // against 3.4 TB/s for the same loads without the non-temporal hint, and 5.5 TB/s for direct-to-VGPR loads in the
@@ -42,8 +40,6 @@
 // result stores issued in between only make that wait stricter, never wrong.
 // Data that crosses workgroups inside the launch uses agent-scope (sc1) loads and stores: an L2-wide write-back /
 // invalidate (__threadfence) per hand-over costs ~4x the whole kernel on this 8-XCD part.
-#include <stdlib.h>
-
 #include <mutex>
 #include <vector>
 
@@ -55,6 +51,7 @@ namespace {
 constexpr int kItemKBlocks = 64;     // most K blocks one UP item covers
 constexpr int kMaxIb = 16;           // most 128-column slices of the intermediate (I <= 2048)
 constexpr int kFinCols = 1024;       // output columns per FIN item
+constexpr int kMaxDynamicLds = 140 << 10;   // of the 160 KiB of a compute unit; the kernel's static tables take ~16 KiB
 
 struct StreamPlan {
     MoeParams p;
@@ -74,30 +71,6 @@ struct StreamPlan {
     int bm_pad;
     int strict_queue;   // every item, the first one too, comes from the counter: correct with any number of resident workgroups
 };
-
-#ifdef ALPHA_MOE_TRACE
-// Debug builds only: per-item timestamps (100 MHz wall clock) for timeline analysis.
-__device__ unsigned long long g_trace[1 << 16][4];
-__device__ int g_trace_n;
-#define TRACE_VARS unsigned long long tr_t0 = 0, tr_t1 = 0
-#define TRACE_BEGIN tr_t0 = tr_t1 = wall_clock64()
-#define TRACE_MARK tr_t1 = wall_clock64()
-#define TRACE_END(kind, idx)                                                                        \
-    if (threadIdx.x == 0) {                                                                         \
-        const int slot_ = atomicAdd(&g_trace_n, 1);                                                 \
-        if (slot_ < (1 << 16)) {                                                                    \
-            g_trace[slot_][0] = ((unsigned long long)(kind) << 56) | ((unsigned long long)blockIdx.x << 32) | (unsigned)(idx); \
-            g_trace[slot_][1] = tr_t0;                                                              \
-            g_trace[slot_][2] = tr_t1;                                                              \
-            g_trace[slot_][3] = wall_clock64();                                                     \
-        }                                                                                           \
-    }
-#else
-#define TRACE_VARS
-#define TRACE_BEGIN
-#define TRACE_MARK
-#define TRACE_END(kind, idx)
-#endif
 
 template <int TM>
 struct Routing {
@@ -134,10 +107,12 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     constexpr int TPK = NT + TM;            // ring tiles per wavefront per K block (token tiles first)
     constexpr int THREADS = WN * 64;
     static_assert(S >= 2 && 2 * (S - 1) < 64, "ring depth must fit the 6-bit vmcnt");
-    // The ring has one slot more than tiles in flight: the load issued at the top of a step then lands in the slot of the
-    // tile read TWO steps ago.  With S slots it would be the tile read one step ago, and a token tile's LDS read (nothing
-    // waits for it until the next matrix instruction) can still be queued when a fast load (the cached dummy line behind the
-    // end of an item) overwrites it: measured as one wavefront's 16 intermediate columns wrong in ~1 of 30 short UP items.
+    // Ring reuse is ordered, not padded: before a load is issued the wavefront waits for all of its own LDS reads
+    // (wait_lds_reads() at the top of every step), so the tile a load overwrites has been read into registers whatever
+    // the ring size.  The hazard this closes: a token tile's LDS read has no consumer until the K block's first matrix
+    // instruction, so with S slots a fast load (the cached dummy line behind the end of an item) could land in the slot
+    // while that read was still queued - seen as one wavefront's 16 intermediate columns wrong in ~1 of 30 short UP
+    // items.  The ring still keeps one slot more than tiles in flight: a load then targets the tile read TWO steps ago.
     constexpr int R = S + 1;
 
     // dynamic LDS: [WN rings of S + 1 tiles][n_ib * TM tiles of requantised activations (DOWN items)]
@@ -148,7 +123,6 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     __shared__ float s_amax[WN][TM * 16];
     __shared__ int s_bcast[2];
 
-    TRACE_VARS;
     const MoeParams &p = s.p;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -176,7 +150,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     const int n_down = n_mb * s.n_cs;
     const int n_fin = p.M * s.n_fc;
     const int total = n_up + n_down + n_fin;
-    const int epoch = __builtin_amdgcn_readfirstlane(s.ctl->epoch) + 1;
+    const int epoch = (int)((unsigned)__builtin_amdgcn_readfirstlane(s.ctl->epoch) + 1u);
     const uint8_t *dummy = p.x;   // where loads past the end of an item are pointed: always mapped, always cached
 
     auto read_tile = [&](const uint8_t *tile) -> v8i {
@@ -319,19 +293,25 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         __syncthreads();   // s_xs is complete
         v8i bfrag[TM];
         for (int kb = 0; kb < nk; kb++) {
-            const float wsg = s_sc[kb], wsu = s_sc[kItemKBlocks + kb];
             float sg[TM], su[TM];
 #pragma unroll
-            for (int t = 0; t < TM; t++) {
-                const float xs = s_xs[t * 16 + n][kb];
-                sg[t] = wsg * xs;
-                su[t] = wsu * xs;
-            }
-#pragma unroll
             for (int a = 0; a < TPK; a++) {
+                // Every LDS read this wavefront has issued is complete before a new direct-to-LDS load may land: a
+                // token tile's read has no consumer until the first matrix instruction of the K block, and nothing
+                // else orders it against the load that re-targets its slot.
+                wait_lds_reads();
                 issue(kb + (a + S - 1) / TPK, (a + S - 1) % TPK, slot_w);
                 slot_w = slot_w + 1 == R ? 0 : slot_w + 1;
                 __builtin_amdgcn_sched_barrier(0);
+                if (a == 0) {   // the K block's scales: read behind the step's load so that their latency hides there
+                    const float wsg = s_sc[kb], wsu = s_sc[kItemKBlocks + kb];
+#pragma unroll
+                    for (int t = 0; t < TM; t++) {
+                        const float xs = s_xs[t * 16 + n][kb];
+                        sg[t] = wsg * xs;
+                        su[t] = wsu * xs;
+                    }
+                }
                 wait_vmcnt<2 * (S - 1)>();
                 const v8i frag = read_tile(ring + slot_r * 2048);
                 slot_r = slot_r + 1 == R ? 0 : slot_r + 1;
@@ -352,7 +332,6 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         }
         fetch_next();
         drain_vmem();
-        TRACE_MARK;
 
         if (s.ks > 1) {
             // K-split: store the valid tokens' partial sums to this item's slice; the last arrival adds the slices up
@@ -383,12 +362,24 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                     v4f g = {0.f, 0.f, 0.f, 0.f}, up = {0.f, 0.f, 0.f, 0.f};
                     if (r.valid[t]) {
                         const float *src = h_u + t * 16 * 256 + my_off + pr * 16;
-                        for (int k = 0; k < s.ks; k++) {   // fixed order: the sum does not depend on arrival order
-                            const v4i gk = ldg128_agent(src + k * slice);
-                            const v4i uk = ldg128_agent(src + k * slice + 128);
-                            drain_vmem();
-                            g += __builtin_bit_cast(v4f, gk);
-                            up += __builtin_bit_cast(v4f, uk);
+                        // fixed order: the sum does not depend on arrival order.  Eight splits (16 loads) are in flight
+                        // at a time: one memory round trip per batch, not per split.
+                        for (int k0 = 0; k0 < s.ks; k0 += 8) {
+                            v4i gk[8], uk[8];
+#pragma unroll
+                            for (int k = 0; k < 8; k++) {
+                                const int kk = k0 + k < s.ks ? k0 + k : s.ks - 1;
+                                gk[k] = ldg128_agent(src + kk * slice);
+                                uk[k] = ldg128_agent(src + kk * slice + 128);
+                            }
+                            drain_vmem_into(gk);
+                            drain_vmem_into(uk);
+#pragma unroll
+                            for (int k = 0; k < 8; k++)
+                                if (k0 + k < s.ks) {
+                                    g += __builtin_bit_cast(v4f, gk[k]);
+                                    up += __builtin_bit_cast(v4f, uk[k]);
+                                }
                         }
                     }
                     accg[pr][t] = g;
@@ -450,10 +441,9 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             // ring after the poll, the others before.
             if (wave != 0) prime();
 
-            if (wave == 0 && !__all(flag0 >= epoch)) spin_all_ge(&s.flag[mb * n_ib], n_ib, epoch, s.ctl);
+            if (wave == 0 && !__all(reached(flag0, epoch))) spin_all_ge(&s.flag[mb * n_ib], n_ib, epoch, s.ctl);
             lds_barrier();   // the flags are up (and s_sc is written); the ring's loads stay in flight
-            TRACE_MARK;
-            if (wave == 0) prime();
+                if (wave == 0) prime();
 
             // requantised activations of all slices -> LDS as operand tiles, their scales -> s_xs[row][ib]
             for (int i = wave; i < n_ib * TM; i += WN) {
@@ -520,13 +510,18 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     auto fin_item = [&](int f) {
         if (tid == 0) spin_until_ge(&s.ctl->down_done, n_down, s.ctl);
         __syncthreads();
-        TRACE_MARK;
         const int t = f / s.n_fc;
         const int c = (f - t * s.n_fc) * kFinCols + tid * 4;
         // lane k fetches the stamp of the token's slot k: one round trip for all of them (top_k <= 64)
         const int stamp = load_agent(&s.live[t * p.top_k + (lane < p.top_k ? lane : 0)]);
+        // A bounded wait that ran out - in this launch or in an earlier one on this workspace: the word is sticky - means
+        // that some result rows may be missing.  The output then says so itself: NaN in every element.
+        const bool poisoned = load_agent(&s.ctl->error) != 0;
         const unsigned long long live_mask = __ballot(lane < p.top_k && stamp == epoch);
-        if (tid < kFinCols / 4 && c < K) {
+        if (poisoned) {
+            if (tid < kFinCols / 4 && c < K)
+                *reinterpret_cast<uint2 *>(p.out + (size_t)t * K + c) = make_uint2(0x7fc07fc0u, 0x7fc07fc0u);
+        } else if (tid < kFinCols / 4 && c < K) {
             v4f sum = {0.f, 0.f, 0.f, 0.f};
             // slot order: the sum depends on nothing but the inputs.  Eight rows are in flight at a time.
             for (int s0 = 0; s0 < p.top_k; s0 += 8) {
@@ -538,7 +533,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                     bits[k] = (v4i){0, 0, 0, 0};
                     if (on) bits[k] = ldg128_agent(s.y + (size_t)slot * K + c);
                 }
-                drain_vmem();
+                drain_vmem_into(bits);
 #pragma unroll
                 for (int k = 0; k < 8; k++) sum += __builtin_bit_cast(v4f, bits[k]);
             }
@@ -561,13 +556,12 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     const int lag = s.lag < n_mb ? s.lag : n_mb;
     const int head_items = lag * per_up;                          // rounds 0 .. lag-1: UP only
     const int mid_items = (n_mb - lag) * (per_up + per_down);     // rounds lag .. n_mb-1: UP then DOWN
-    auto run_item = [&](int item) -> int {
+    // every item kind has exactly one call site: the compiler inlines the item bodies into the loop
+    auto run_item = [&](int item) {
+        int up = -1, down = -1, fin = -1;
         if (item >= n_up + n_down) {
-            fin_item(item - n_up - n_down);
-            return 3;
-        }
-        int up = -1, down = -1;
-        if (item < head_items) {
+            fin = item - n_up - n_down;
+        } else if (item < head_items) {
             up = item;
         } else if (item < head_items + mid_items) {
             const int i = item - head_items;
@@ -580,12 +574,9 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         } else {
             down = (n_mb - lag) * per_down + (item - head_items - mid_items);
         }
-        if (up >= 0) {
-            up_item(up);
-            return 1;
-        }
-        down_item(down);
-        return 2;
+        if (up >= 0) up_item(up);
+        else if (down >= 0) down_item(down);
+        else fin_item(fin);
     };
     int item = blockIdx.x;   // no round trip to the queue before the first item
     if (s.strict_queue) {    // unless the caller cannot promise that the whole grid is resident at once
@@ -596,13 +587,10 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         __syncthreads();
     }
     while (item < total) {
-        TRACE_BEGIN;
         next_item = -1;
-        const int kind = run_item(item);
-        (void)kind;
+        run_item(item);
         fetch_next();   // paths that did not get there themselves (skipped blocks, FIN items)
         __syncthreads();
-        TRACE_END(kind, item);
         if (tid == 0) s_bcast[0] = next_item;
         __syncthreads();
         item = __builtin_amdgcn_readfirstlane(s_bcast[0]);
@@ -620,14 +608,8 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
 
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 
-int env_int(const char *name, int dflt)
-{
-    const char *e = getenv(name);
-    return e ? atoi(e) : dflt;
-}
-
-// Everything the host decides about one launch; a pure function of the sizes (and of the tuning overrides in the
-// environment), so the workspace query and the launch agree.
+// Everything the host decides about one launch; a pure function of the sizes (and of the tuning overrides), so the
+// workspace query and the launch agree.
 struct HostPlan {
     bool ok;
     int bm_pad, n_ib, nkb, n_ct, n_mb_max, units;
@@ -678,7 +660,7 @@ HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int bl
     if (ks_want < 1) ks_want = 1;
     int kbpi = (h.nkb + ks_want - 1) / ks_want;
     if (kbpi < 4) kbpi = 4;
-    kbpi = env_int("ALPHA_MOE_KBPI", kbpi);
+    kbpi = tunable(kTunKbpi, kbpi);
     if (kbpi < 1) kbpi = 1;
     if (kbpi > h.nkb) kbpi = h.nkb;
     if (kbpi > kItemKBlocks) kbpi = kItemKBlocks;
@@ -691,7 +673,7 @@ HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int bl
     // small experts, about a row block per compute unit: one DOWN item per block (Qwen3-Next shard, M = 32: -7 %)
     if ((int64_t)h.n_ct * 2048 * h.n_ib <= (512 << 10) && mb_est * 4 >= cus * 3) down_target = 512 << 10;
     int tpi = (int)(down_target / (2048 * h.n_ib)) / 16 * 16;
-    tpi = env_int("ALPHA_MOE_TPI", tpi);
+    tpi = tunable(kTunTpi, tpi);
     if (tpi < 16) tpi = 16;
     tpi = (tpi + 15) / 16 * 16;
     if (tpi > (h.n_ct + 15) / 16 * 16) tpi = (h.n_ct + 15) / 16 * 16;
@@ -703,7 +685,7 @@ HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int bl
     // how many row blocks later a block's DOWN items enter the queue than its UP items
     // (measured: overlapping the two kinds lowers the total rate - DOWN items stream less efficiently than UP items -
     // so by default the lag is "all blocks", i.e. UP items first, then DOWN items)
-    h.lag = env_int("ALPHA_MOE_LAG", 1 << 30);
+    h.lag = tunable(kTunLag, 1 << 30);
     if (h.lag < 1) h.lag = 1;
 
     size_t off = align_up(kPrefixBytes);
@@ -779,7 +761,7 @@ hipError_t resident_slots(const Variant &v, int lds_bytes, int *slots)
     err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     if (err != hipSuccess) return err;
     err = hipFuncSetAttribute(reinterpret_cast<const void *>(v.fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              128 << 10);
+                              kMaxDynamicLds);
     if (err != hipSuccess) return err;
     int occ = 0;
     err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, reinterpret_cast<const void *>(v.fn), v.threads,
@@ -804,21 +786,6 @@ hipError_t resident_slots(const Variant &v, int lds_bytes, int *slots)
 }
 
 }  // namespace
-
-#ifdef ALPHA_MOE_TRACE
-extern "C" int alpha_moe_debug_trace_read(void *dst, int max_records)
-{
-    int n = 0;
-    (void)hipDeviceSynchronize();
-    (void)hipMemcpyFromSymbol(&n, HIP_SYMBOL(g_trace_n), sizeof(int));
-    if (n > max_records) n = max_records;
-    if (n > (1 << 16)) n = 1 << 16;
-    (void)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_trace), (size_t)n * 32);
-    const int zero = 0;
-    (void)hipMemcpyToSymbol(HIP_SYMBOL(g_trace_n), &zero, sizeof(int));
-    return n;
-}
-#endif
 
 size_t stream_prefix_bytes() { return align_up(kPrefixBytes); }
 
@@ -858,16 +825,25 @@ hipError_t launch_stream(const MoeParams &p, int warp_n, int stages, void *works
     s.n_cs = h.n_cs;
     s.n_fc = h.n_fc;
     s.lag = h.lag;
-    s.strict_queue = env_int("ALPHA_MOE_STRICT_QUEUE", 0) != 0;
+    s.strict_queue = tunable(kTunStrictQueue, 1) != 0;
 
-    const Variant v = pick((p.block_m + 15) / 16, warp_n, stages);
-    const int lds_bytes = v.ring_bytes + h.n_ib * v.tm * 2048;
+    // `stages` asks for a ring depth; what LDS holds next to the item tables decides.  The shallowest ring always fits.
+    const int tm = (p.block_m + 15) / 16;
+    const int tail_bytes = h.n_ib * tm * 2048;   // DOWN items: the requantised tiles of all slices
+    Variant v = pick(tm, warp_n, stages);
+    int lds_bytes = v.ring_bytes + tail_bytes;
+    while (lds_bytes > kMaxDynamicLds && stages > 1) {
+        stages--;
+        v = pick(tm, warp_n, stages);
+        lds_bytes = v.ring_bytes + tail_bytes;
+    }
+    if (lds_bytes > kMaxDynamicLds) return hipErrorInvalidValue;
     int slots = 0;
     const hipError_t err = resident_slots(v, lds_bytes, &slots);
     if (err != hipSuccess) return err;
 
     const int64_t max_items = (int64_t)h.units * h.ks + (int64_t)h.n_mb_max * h.n_cs + (int64_t)p.M * h.n_fc;
-    int grid = env_int("ALPHA_MOE_GRID", slots);
+    int grid = tunable(kTunGrid, slots);
     if (grid > max_items) grid = (int)max_items;
     if (grid < 1) grid = 1;
     hipLaunchKernelGGL(v.fn, dim3((unsigned)grid), dim3((unsigned)v.threads), lds_bytes, stream, s);

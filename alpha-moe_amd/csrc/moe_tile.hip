@@ -33,8 +33,7 @@
 // blocks (one workgroup per block left 16 of 272 blocks at M = 1024 to a second round: 547 us, now 391 us), the
 // blocks of one expert next to each other on one XCD so that they share its L2, and non-temporal loads for the
 // weights of experts that have a single block.
-#include <stdlib.h>
-
+#include <mutex>
 #include <type_traits>
 
 #include "moe_common.hpp"
@@ -150,7 +149,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
     const int q = lane >> 4;
     const int K = p.K, I = p.N >> 1;
     const int n_ib = s.n_ib, nkb = s.nkb;
-    const int epoch = __builtin_amdgcn_readfirstlane(s.ctl->epoch) + 1;
+    const int epoch = (int)((unsigned)__builtin_amdgcn_readfirstlane(s.ctl->epoch) + 1u);
     uint8_t *a_ring = lds_dyn + w * (kStages * 8192);
     uint8_t *xbuf = lds_dyn + kARingBytes;
 
@@ -524,7 +523,10 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
 __global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams s, int chunks_per_token, int n_units)
 {
     const MoeParams &p = s.p;
-    const int epoch = s.ctl->epoch + 1;
+    const int epoch = (int)((unsigned)s.ctl->epoch + 1u);
+    // a bounded wait that ran out (in this call's tile kernel or in any earlier launch on this workspace: the word is
+    // sticky) means result rows may be missing: the output then says so itself, NaN in every element
+    const bool poisoned = load_agent(&s.ctl->error) != 0;
     for (int unit = blockIdx.x; unit < n_units; unit += gridDim.x) {
         const int t = unit / chunks_per_token;
         const int c = (unit - t * chunks_per_token) * 2048 + threadIdx.x * 8;
@@ -557,7 +559,7 @@ __global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams s
         add(prior);
         v4i o;
 #pragma unroll
-        for (int i = 0; i < 4; i++) o[i] = (int)pack_bf16x2(sum[2 * i], sum[2 * i + 1]);
+        for (int i = 0; i < 4; i++) o[i] = poisoned ? 0x7fc07fc0 : (int)pack_bf16x2(sum[2 * i], sum[2 * i + 1]);
         *op = o;
     }
     __syncthreads();
@@ -571,12 +573,6 @@ __global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams s
 }
 
 size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
-
-int env_int(const char *name, int dflt)
-{
-    const char *e = getenv(name);
-    return e ? atoi(e) : dflt;
-}
 
 // Token parts of a DOWN item: the smallest divisor nh of th such that the requantised tiles of all n_ib slices of a
 // part (2 th / nh tiles per slice) fit next to the weight rings; 0 if none does.
@@ -609,13 +605,29 @@ TileFn pick(int th)
     }
 }
 
+// The variant's dynamic LDS limit is raised once per (variant, device), not on every launch.
+hipError_t allow_dynamic_lds(int th, TileFn fn)
+{
+    static std::mutex mu;
+    static bool done[5][64];
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return err;
+    std::lock_guard<std::mutex> lock(mu);
+    if (dev >= 0 && dev < 64 && done[th][dev]) return hipSuccess;
+    err = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
+                              kARingBytes + kMaxTailBytes);
+    if (err == hipSuccess && dev >= 0 && dev < 64) done[th][dev] = true;
+    return err;
+}
+
 }  // namespace
 
 // 64-column groups per DOWN item: about 14 ring steps (a step is one group x one slice), a multiple of 4 so that
 // every pair of wavefronts gets the same number of groups
 static int groups_per_item(int n_ib)
 {
-    const int e = env_int("ALPHA_MOE_TILE_GPS", 0);
+    const int e = tunable(kTunTileGps, 0);
     if (e > 0) return (e + 3) / 4 * 4;
     return 4 * ((14 + n_ib - 1) / n_ib);
 }
@@ -661,14 +673,13 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
     s.n_cs = ((p.K >> 6) + s.gps - 1) / s.gps;
     // up/gate items of this many row blocks run ahead of the first down items of a queue: with ~32 workgroups
     // on a queue, a down item's up/gate items were taken at least two rounds of the queue earlier
-    s.lag = env_int("ALPHA_MOE_TILE_LAG", 64);
-    s.w_nt = env_int("ALPHA_MOE_TILE_NT", -1);
+    s.lag = tunable(kTunTileLag, 64);
+    s.w_nt = tunable(kTunTileNt, -1);
     if (s.lag < 1) s.lag = 1;
     const TileFn fn = pick(tm / 2);
     s.nh = token_parts(tm / 2, s.n_ib);
     const int lds_bytes = kARingBytes + tail_bytes(tm / 2, s.n_ib);
-    hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void *>(fn), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         kARingBytes + kMaxTailBytes);
+    hipError_t err = allow_dynamic_lds(tm / 2, fn);   // once per variant and device
     if (err != hipSuccess) return err;
     // persistent workgroups, one per compute unit (the rings take most of a CU's LDS); fewer when there is less work
     static const int cus = [] {
@@ -679,7 +690,7 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
         return n;
     }();
     const int64_t items = (int64_t)s.n_mb_max * (s.n_ib + s.n_cs * s.nh);
-    int grid = env_int("ALPHA_MOE_TILE_GRID", cus);
+    int grid = tunable(kTunTileGrid, cus);
     if (grid > items) grid = (int)((items + 7) / 8 * 8);
     if (grid < 8) grid = 8;
     hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(512), lds_bytes, stream, s);

@@ -14,31 +14,70 @@
 
 #include "../../include/alpha_moe_hip.h"
 
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
 #include <map>
-#include <tuple>
 #include <mutex>
+#include <tuple>
 #include <utility>
+#include <vector>
 
 namespace {
 
 // Scratch for the C ABI, one buffer per (device, stream): zero-filled when created and maintained by the library
-// afterwards, so the steady state allocates and clears nothing (the first call on a stream, or the first with a
-// larger problem, does both: warm the operator up once before capturing it into a HIP graph).
+// afterwards, so the steady state allocates and clears nothing.  A buffer is never freed or shrunk once a call has
+// used it: a HIP graph captured earlier may hold its address, and its replays keep writing the control block, flags
+// and result rows there.  When a later call needs more, a new buffer of exactly that size takes over for eager calls
+// and the old one stays alive beside it (graphs captured before keep replaying into it).  Growth while the stream is
+// being captured is refused: the fill of the new buffer's control prefix would be recorded into the graph and run on
+// every replay, and the allocation would belong to the graph's private pool.  reserve_workspace() sizes the buffer
+// ahead of time.
+struct StreamScratch {
+    at::Tensor current;
+    std::vector<at::Tensor> retired;
+};
+
 at::Tensor workspace_for(const at::Device &dev, hipStream_t stream, size_t bytes)
 {
     static std::mutex mu;
-    static std::map<std::pair<int, void *>, at::Tensor> cache;
+    static std::map<std::pair<int, void *>, StreamScratch> cache;
     std::lock_guard<std::mutex> lock(mu);
-    at::Tensor &slot = cache[{dev.index(), static_cast<void *>(stream)}];
-    if (!slot.defined() || static_cast<size_t>(slot.numel()) < bytes) {
-        size_t cap = 1 << 20;
-        while (cap < bytes) cap <<= 1;
-        slot = at::empty({static_cast<int64_t>(cap)}, at::TensorOptions().dtype(at::kByte).device(dev));
-        // only the control block, counters and flags have to start at zero (1.5 MiB, not the whole buffer: under HIP
-        // graph capture this fill is recorded and runs on every replay)
-        slot.narrow(0, 0, static_cast<int64_t>(alpha_moe_workspace_zero_bytes())).zero_();
+    StreamScratch &slot = cache[{dev.index(), static_cast<void *>(stream)}];
+    if (!slot.current.defined() || static_cast<size_t>(slot.current.numel()) < bytes) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        (void)hipStreamIsCapturing(stream, &capturing);
+        TORCH_CHECK(capturing == hipStreamCaptureStatusNone,
+                    "alpha_moe: this call needs ", bytes, " bytes of scratch memory on a stream that is being captured "
+                    "and holds ", slot.current.defined() ? slot.current.numel() : 0, ": run the operator once with "
+                    "these sizes before the capture, or call torch.ops.alpha_moe.reserve_workspace(x, bytes) there");
+        if (slot.current.defined()) slot.retired.push_back(slot.current);
+        const size_t cap = (bytes + 255) & ~static_cast<size_t>(255);
+        slot.current = at::empty({static_cast<int64_t>(cap)}, at::TensorOptions().dtype(at::kByte).device(dev));
+        // only the control block, counters and flags have to start at zero (1.5 MiB, not the whole buffer)
+        slot.current.narrow(0, 0, static_cast<int64_t>(alpha_moe_workspace_zero_bytes())).zero_();
     }
-    return slot;
+    return slot.current;
+}
+
+// reserve_workspace(like, bytes): make the scratch buffer of (like's device, the current stream) at least `bytes`
+// large now, e.g. alpha_moe_workspace_bytes() of the largest call a graph captured later on this stream will make.
+void reserve_workspace(const at::Tensor &like, int64_t bytes)
+{
+    TORCH_CHECK(like.is_cuda(), "reserve_workspace: `like` must be a GPU tensor (it names the device)");
+    TORCH_CHECK(bytes >= 0, "reserve_workspace: bytes must not be negative");
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(like.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    const size_t need = std::max(static_cast<size_t>(bytes), alpha_moe_workspace_zero_bytes());
+    (void)workspace_for(like.device(), stream, need);
+}
+
+// bytes of scratch a call with these sizes needs (alpha_moe_workspace_bytes of the C ABI)
+int64_t workspace_bytes(int64_t top_k, int64_t M, int64_t K, int64_t N, int64_t E, int64_t sorted_num, int64_t block_m)
+{
+    return static_cast<int64_t>(alpha_moe_workspace_bytes(static_cast<int>(top_k), static_cast<int>(M), static_cast<int>(K),
+                                                          static_cast<int>(N), static_cast<int>(E),
+                                                          static_cast<int>(sorted_num), static_cast<int>(block_m)));
 }
 
 void check_tensor(const at::Tensor &t, const char *name, at::ScalarType dtype, const at::Device &dev)
@@ -195,6 +234,9 @@ TORCH_LIBRARY_FRAGMENT(alpha_moe, m)
     m.impl("per_token_group_quant_fp8", c10::DispatchKey::CUDA, &per_token_group_quant_fp8);
     m.def("moe_align_block_size(Tensor topk_ids, int block_size, int num_experts) -> (Tensor, Tensor, Tensor)");
     m.impl("moe_align_block_size", c10::DispatchKey::CUDA, &moe_align_block_size);
+    m.def("reserve_workspace(Tensor like, int bytes) -> ()");
+    m.impl("reserve_workspace", c10::DispatchKey::CUDA, &reserve_workspace);
+    m.def("workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m) -> int", &workspace_bytes);
     m.def("fused_moe_w8a8_up_down("
           "Tensor x, Tensor x_scale, Tensor w, Tensor w_scale, Tensor w2, Tensor w2_scale, "
           "Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_post_padded, Tensor topk_weights, "

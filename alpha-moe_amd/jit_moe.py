@@ -51,12 +51,12 @@ def bench_events(fn, num_tests: int = 25, flush_bytes: int = 512 << 20):
 
 
 def generate_topk_ids(num_experts, num_tokens, top_k, balancedness=1.0):
-    """Expert ids drawn with replacement from balancedness * uniform + (1 - balancedness) * (all on expert 0)."""
-    uniform = torch.ones(num_experts) / num_experts
-    skewed = torch.zeros(num_experts)
-    skewed[0] = 1.0
-    probs = balancedness * uniform + (1 - balancedness) * skewed
-    ids = torch.multinomial(probs, num_tokens * top_k, replacement=True)
+    """Routing for the sweep: every slot independently goes to a uniformly drawn expert with probability
+    `balancedness` and to expert 0 otherwise (the mixture the reference's generator draws from, jit_moe.py:34-51;
+    a token may name an expert twice, as there)."""
+    n_slots = num_tokens * top_k
+    ids = torch.randint(0, num_experts, (n_slots,))
+    ids[torch.rand(n_slots) >= balancedness] = 0
     return ids.view(num_tokens, top_k)
 
 

@@ -9,7 +9,10 @@ resident in HBM.  The headline is M=64 decode against the HBM roofline; the same
 sizes of that shard (decode M = 1, 4, 16 and prefill M = 512, 2048, 8192, reported under "per_M" with both the HBM and
 the FP8 MFMA fraction) and the Qwen3-Next-like and Qwen3-30B-like shards ("other_configs").
 Consecutive steps rotate through several copies of the weights and several routings so that a step never finds its
-weights in the 256 MiB Infinity Cache; `out` is not re-zeroed inside the timed region (the operator adds into it).
+weights in the 256 MiB Infinity Cache; where that rotation touches less than 1 GiB (small M), every timed call is
+preceded by a 512 MiB fill that evicts L2 and the Infinity Cache, and the figure is the mean of the per-call device
+times ("cold": true).  `out` is not re-zeroed inside the timed region (the operator adds into it).
+Every reported size is also checked against the CPU oracle on a sample of its tokens ("parity_sample").
 
 Prints ONE JSON line: the driver's contract fields plus
   "roofline":     algorithmic HBM bytes per launch / average launch duration (HIP events on the launch stream)
@@ -50,6 +53,7 @@ def parse_args():
     ap.add_argument("--replicas", type=int, default=6, help="copies of the weights rotated through")
     ap.add_argument("--config", default=None, help="tuning table (JSON of jit_moe.py); default: shipped table or built-in knobs")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity-samples", action="store_true", help="skip the oracle check of every reported size")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy three times: a kernel of known traffic to scale "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings by")
@@ -74,6 +78,11 @@ def main():
     dev = "cuda:0"
     torch.cuda.set_device(0)
     n_routings = 8
+
+    flush_buf = torch.empty((512 << 20) // 4, dtype=torch.int32, device=dev)
+
+    def flush_caches(i):
+        flush_buf.fill_(i)   # 512 MiB written: nothing of an earlier call is left in L2 or the Infinity Cache
 
     class Bench:
         """Weights of one shape (rotated copies) and the measurement of one batch size on them."""
@@ -112,10 +121,43 @@ def main():
                         P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids, total, P.topk_weights, out,
                         s.top_k, knobs["block_m"], knobs["block_n"], knobs["warp_n"], knobs["stages"], s.scaling_factor)
                 calls.append(call)
+            self.last = (P, W, s_ids, e_ids, total, out, knobs)
             return calls, statistics.mean(byts), statistics.mean(flops), knobs, src
+
+        def parity_sample(self, n=12):
+            """The last prepared problem's output rows for a sample of its tokens against the CPU oracle on those tokens
+            alone (a token's result depends only on its own row, routing and the weights)."""
+            from oracle import moe_oracle as O
+            from alpha_moe_python.workloads import Problem
+            P, W, s_ids, e_ids, total, out, knobs = self.last
+            s = self.shape
+            out.zero_()
+            torch.ops.alpha_moe.fused_moe_w8a8_up_down(
+                P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids, total, P.topk_weights, out,
+                s.top_k, knobs["block_m"], knobs["block_n"], knobs["warp_n"], knobs["stages"], s.scaling_factor)
+            torch.cuda.synchronize()
+            idx = torch.randperm(P.M, generator=torch.Generator().manual_seed(5))[:n].sort().values
+            sub = Problem(W, len(idx), P.x[idx.to(dev)].contiguous(), P.x_scale[idx.to(dev)].contiguous(),
+                          P.topk_ids[idx.to(dev)].contiguous(), P.topk_weights[idx.to(dev)].contiguous())
+            ids = sub.align(16)
+            # only the sample's experts cross to the host
+            used = torch.unique(sub.topk_ids).long()
+            remap = torch.full((s.E,), -1, dtype=torch.int32, device=dev)
+            remap[used] = torch.arange(len(used), dtype=torch.int32, device=dev)
+            e_sub = torch.where(ids[1] >= 0, remap[ids[1].clamp(min=0).long()], ids[1])
+            ref = O.fused_moe_oracle(sub.x.cpu(), sub.x_scale.cpu(), W.w1[used].cpu(), W.w1_scale[used].cpu(),
+                                     W.w2[used].cpu(), W.w2_scale[used].cpu(), ids[0].cpu(), e_sub.cpu(), ids[2].cpu(),
+                                     sub.topk_weights.cpu(), torch.zeros((len(idx), s.K), dtype=torch.bfloat16),
+                                     s.top_k, 16, s.scaling_factor)
+            m = O.error_metrics(out[idx.to(dev)], ref)
+            return {"tokens": len(idx), "max_abs_over_max_ref": round(m["max_abs_over_max_ref"], 5),
+                    "cosine": round(m["cosine"], 7),
+                    "ok": bool(m["max_abs_over_max_ref"] <= 1e-2 and m["cosine"] >= 0.9999)}
 
         def measure(self, M, steps, warmup):
             calls, B, F, knobs, src = self.prepare(M)
+            # does the rotation alone keep a step's weights out of the 256 MiB Infinity Cache?
+            cold = B * len(calls) < (1 << 30)
             for i in range(warmup):
                 calls[i % len(calls)]()
             torch.cuda.synchronize()
@@ -127,18 +169,30 @@ def main():
             # per-launch device time: HIP events on the launch stream (torch's current stream) around every call
             evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
             for i in range(steps):
+                if cold:
+                    flush_caches(i)
                 evs[i][0].record()
                 calls[i % len(calls)]()
                 evs[i][1].record()
             torch.cuda.synchronize()
             dev_ms = [a.elapsed_time(b) for a, b in evs]
-            return {"M": M, "ms_per_step": wall_ms, "launch_us_mean": statistics.mean(dev_ms) * 1e3,
-                    "launch_us_median": statistics.median(dev_ms) * 1e3, "launch_us_min": min(dev_ms) * 1e3,
-                    "bytes": B, "flops": F, "knobs": knobs, "knobs_from": src}
+            r = {"M": M, "ms_per_step": wall_ms, "launch_us_mean": statistics.mean(dev_ms) * 1e3,
+                 "launch_us_median": statistics.median(dev_ms) * 1e3, "launch_us_min": min(dev_ms) * 1e3,
+                 "bytes": B, "flops": F, "knobs": knobs, "knobs_from": src, "cold": cold}
+            if not args.no_parity_samples:
+                r["parity_sample"] = self.parity_sample()
+            return r
 
     def summarise(r):
         t_us = r["launch_us_mean"]
-        return {"us_per_layer": round(r["ms_per_step"] * 1e3, 2), "launch_us_mean": round(t_us, 2),
+        # cold rows: the wall-clock rotation may find its weights in the Infinity Cache, the flushed launches do not
+        us_layer = t_us if r["cold"] else r["ms_per_step"] * 1e3
+        extra = {"cold": r["cold"]}
+        if r["cold"]:
+            extra["us_per_layer_rotation_only"] = round(r["ms_per_step"] * 1e3, 2)
+        if "parity_sample" in r:
+            extra["parity_sample"] = r["parity_sample"]
+        return {"us_per_layer": round(us_layer, 2), "launch_us_mean": round(t_us, 2), **extra,
                 "launch_us_median": round(r["launch_us_median"], 2),
                 "algorithmic_MB": round(r["bytes"] / 1e6, 1), "GB_per_s": round(r["bytes"] / t_us / 1e3, 1),
                 "hbm_frac": round(r["bytes"] / t_us / 1e3 / HBM_PEAK_GBS, 4),

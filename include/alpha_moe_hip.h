@@ -102,7 +102,8 @@ size_t alpha_moe_workspace_zero_bytes(void);
  * workspace a workgroup gave up waiting for another (each such wait is bounded at a few seconds so that nothing
  * hangs; the results of that launch are not valid), ALPHA_MOE_OK otherwise.  The flag is sticky until the prefix is
  * zero-filled again.  Synchronises, so it is for tests and health checks, not for the serving loop.  The reference's
- * kernel has no waits between thread blocks and no counterpart.
+ * kernel has no waits between thread blocks and no counterpart.  Callers need not poll it to notice: while the flag
+ * is set, every call on the workspace fills `out` with NaN.
  */
 int alpha_moe_workspace_check(const void *workspace, void *stream /* hipStream_t */);
 
@@ -142,6 +143,16 @@ int alpha_moe_moe_align_block_size(const int32_t *topk_ids, int numel, int num_e
                                    int32_t *sorted_token_ids, int sorted_num, int32_t *expert_ids, int n_blocks,
                                    int32_t *num_tokens_post_padded, void *workspace, size_t workspace_bytes,
                                    void *stream /* hipStream_t */);
+
+/*
+ * Tuning overrides, for experiments and tests: `name` is one of ALPHA_MOE_PATH (1 direct, 2 stream, 3 tile),
+ * ALPHA_MOE_STRICT_QUEUE, ALPHA_MOE_KBPI, ALPHA_MOE_TPI, ALPHA_MOE_LAG, ALPHA_MOE_GRID,
+ * ALPHA_MOE_TILE_GPS, ALPHA_MOE_TILE_LAG, ALPHA_MOE_TILE_GRID, ALPHA_MOE_TILE_NT.  set != 0 installs `value`, set == 0
+ * returns the choice to the library.  The environment variables of the same names are read once, when the library is
+ * first used; no launch reads the environment.  Not thread-safe against concurrent launches.  Results stay within
+ * the parity bar whatever is set.  Returns ALPHA_MOE_ERR_SHAPE for an unknown name.  No counterpart in the reference.
+ */
+int alpha_moe_set_tunable(const char *name, int value, int set);
 
 /* Human-readable text for a status code (static storage). */
 const char *alpha_moe_status_string(int status);

@@ -1,5 +1,7 @@
 """Shared helpers of the GPU parity tests: run the operator (through torch.ops or straight through the C ABI)
 and the CPU oracle on the same bits."""
+import contextlib
+
 import torch
 
 from oracle import moe_oracle as O
@@ -56,3 +58,27 @@ def assert_parity(out, ref, what=""):
     assert torch.isfinite(out.float()).all(), what
     assert m["max_abs_over_max_ref"] <= MAX_ABS_OVER_MAX_REF and m["cosine"] >= MIN_COSINE, (what, m)
     return m
+
+
+@contextlib.contextmanager
+def tunables(**values):
+    """Tuning overrides of the library for the duration of a with-block: tunables(ALPHA_MOE_TILE_GRID=8)."""
+    import alpha_moe
+    for name, value in values.items():
+        alpha_moe.set_tunable(name, value)
+    try:
+        yield
+    finally:
+        for name in values:
+            alpha_moe.set_tunable(name, None)
+
+
+def sampled_tokens_match_oracle(P, out, what, n=48, seed=11):
+    """A token's result depends on nothing but its own row, routing and the weights: the oracle recomputes a random
+    sample of the tokens as an n-token problem of its own."""
+    from alpha_moe_python.workloads import Problem
+    gen = torch.Generator().manual_seed(seed)
+    idx = torch.randperm(P.M, generator=gen)[:n].sort().values.to(P.x.device)
+    sub = Problem(P.weights, n, P.x[idx].contiguous(), P.x_scale[idx].contiguous(), P.topk_ids[idx].contiguous(),
+                  P.topk_weights[idx].contiguous())
+    return assert_parity(out[idx], oracle_out(sub), what)

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from alpha_moe_python.workloads import SHAPES, Shape, make_problem, make_weights
-from gpu_util import assert_parity, oracle_out, run_op
+from gpu_util import assert_parity, oracle_out, run_op, sampled_tokens_match_oracle, tunables
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -195,6 +195,19 @@ def test_deepseek_shard_prefill_full_size_properties(ds_weights):
     assert torch.equal(out, run_op(P, 64, 64, 4, 3, via="c_abi"))
 
 
+@pytest.mark.parametrize("M,knobs", [(512, (64, 64, 4, 3)), (2048, (96, 64, 4, 3))])
+def test_deepseek_shard_prefill_mid_sizes(ds_weights, M, knobs):
+    """The two mid prefill sizes of the DeepSeek-V3 shard with the knobs of the shipped tuning table: sampled tokens
+    against the oracle (a token's result depends only on its own row, routing and the weights), and a second launch
+    bit for bit."""
+    P = make_problem(ds_weights, M, seed=3)
+    print(f"case ds M={M} knobs {knobs}", flush=True)
+    out = run_op(P, *knobs, via="c_abi")
+    print("metrics", sampled_tokens_match_oracle(P, out, f"ds M={M} sampled tokens"), flush=True)
+    print(f"case ds M={M} second launch", flush=True)
+    assert torch.equal(out, run_op(P, *knobs, via="c_abi"))
+
+
 def _sampled_tokens_match_oracle(P, out, what, n=48, seed=11):
     """A token's result depends on nothing but its own row, routing and the weights: recompute a sample on the CPU."""
     from alpha_moe_python.workloads import Problem
@@ -243,6 +256,17 @@ def test_qwen3_30b_zipf_shard_against_oracle(q3_weights, M, knobs):
     print("metrics", m, flush=True)
 
 
+def test_qwen3_30b_zipf_shard_prefill_M1024(q3_weights):
+    """M=1024 of the Zipf shard with the shipped table's knobs: the hot experts have many row blocks, most have one."""
+    P = make_problem(q3_weights, 1024, seed=2)
+    knobs = (64, 64, 4, 3)
+    print(f"case q3 M=1024 knobs {knobs}", flush=True)
+    out = run_op(P, *knobs, via="c_abi")
+    print("metrics", sampled_tokens_match_oracle(P, out, "q3 M=1024 sampled tokens"), flush=True)
+    print("case q3 M=1024 second launch", flush=True)
+    assert torch.equal(out, run_op(P, *knobs, via="c_abi"))
+
+
 def test_qwen3_30b_zipf_shard_prefill_full_size(q3_weights):
     P = make_problem(q3_weights, 8192, seed=1)
     print("case q3 M=8192 knobs (64, 32, 8, 3)", flush=True)
@@ -261,7 +285,8 @@ def test_short_up_items_repeat_launches():
     W = make_weights(shape, device=DEV, seed=0)
     P = make_problem(W, 32, seed=0)
     ref = oracle_out(P)
-    for knobs in ((16, 32, 8, 5), (16, 32, 8, 2), (16, 64, 4, 1), (16, 64, 4, 2)):
+    for knobs in ((16, 32, 8, 5), (16, 32, 8, 2), (16, 64, 4, 1), (16, 64, 4, 2),
+                  (32, 32, 8, 5), (32, 64, 4, 2), (24, 32, 8, 3)):   # the last three: two token tiles per row block
         print(f"case short M=32 knobs {knobs}", flush=True)
         first = run_op(P, *knobs, via="c_abi")
         assert_parity(first, ref, f"short M=32 knobs {knobs}")
@@ -287,7 +312,7 @@ def test_grid_fits_the_device(ds_weights, knobs):
     assert_parity(out, oracle_out(P), f"ds M=64 knobs {knobs}")
 
 
-def test_tile_kernel_result_independent_of_item_schedule(monkeypatch):
+def test_tile_kernel_result_independent_of_item_schedule():
     """The tile kernel's work items (up/gate slices, slabs of output columns) may run on any workgroup in any order
     that respects their flags: few workgroups (every one serves all eight queues), down items right behind their
     up/gate items, the smallest and the largest column slabs, cached or non-temporal weight loads - the output is
@@ -298,19 +323,15 @@ def test_tile_kernel_result_independent_of_item_schedule(monkeypatch):
     W = make_weights(shape, device=DEV, seed=3)
     P = make_problem(W, 300, seed=3)
     ref = oracle_out(P)
-    for name in ("ALPHA_MOE_TILE_GRID", "ALPHA_MOE_TILE_LAG", "ALPHA_MOE_TILE_GPS", "ALPHA_MOE_TILE_NT"):
-        monkeypatch.delenv(name, raising=False)
     for block_m in (48, 128):
         print(f"case sched M=300 block_m {block_m} default schedule", flush=True)
         base = run_op(P, block_m, 64, 4, 3, via="c_abi")
         assert_parity(base, ref, f"sched block_m {block_m}")
-        for env in ({"ALPHA_MOE_TILE_GRID": "8"}, {"ALPHA_MOE_TILE_LAG": "1"}, {"ALPHA_MOE_TILE_GPS": "4"},
-                    {"ALPHA_MOE_TILE_GPS": "1000"}, {"ALPHA_MOE_TILE_NT": "1"}, {"ALPHA_MOE_TILE_NT": "0"},
-                    {"ALPHA_MOE_TILE_GRID": "16", "ALPHA_MOE_TILE_LAG": "2", "ALPHA_MOE_TILE_GPS": "8"}):
+        for env in ({"ALPHA_MOE_TILE_GRID": 8}, {"ALPHA_MOE_TILE_LAG": 1}, {"ALPHA_MOE_TILE_GPS": 4},
+                    {"ALPHA_MOE_TILE_GPS": 1000}, {"ALPHA_MOE_TILE_NT": 1}, {"ALPHA_MOE_TILE_NT": 0},
+                    {"ALPHA_MOE_TILE_GRID": 16, "ALPHA_MOE_TILE_LAG": 2, "ALPHA_MOE_TILE_GPS": 8}):
             print(f"case sched M=300 block_m {block_m} {env}", flush=True)
-            with monkeypatch.context() as mp:
-                for k, v in env.items():
-                    mp.setenv(k, v)
+            with tunables(**env):
                 got = run_op(P, block_m, 64, 4, 3, via="c_abi")
             assert torch.equal(got, base), (block_m, env)
 
@@ -444,33 +465,45 @@ def test_workspace_check_reports_an_expired_wait(c1):
     ws.view(torch.int32)[3] = 1   # the control block's error word
     rc = alpha_moe.c_abi.alpha_moe_workspace_check(ws.data_ptr(), stream)
     assert rc == 8 and b"wait" in alpha_moe.c_abi.alpha_moe_status_string(rc)
+    # while the word is set, every call on the workspace says so in its output: NaN everywhere, adding or storing,
+    # from the streaming kernel and from the tile kernel
+    for knobs in ((16, 32, 8, 5), (64, 64, 4, 3)):
+        for store in (False, True):
+            got = run_op(P, *knobs, via="c_abi", workspace=ws, store=store)
+            assert torch.isnan(got.float()).all(), (knobs, store)
+    ws.view(torch.int32)[3] = 0
+    assert_parity(run_op(P, 16, 32, 8, 5, via="c_abi", workspace=ws), ref, "after clearing the error word")
 
 
-def test_strict_queue_survives_a_grid_the_device_cannot_hold(ds_weights, monkeypatch):
-    """With ALPHA_MOE_STRICT_QUEUE=1 no workgroup owns an item before it runs, so even a grid of four times what the
-    device holds at once (workgroups that start only when others have left) finishes at once and correctly - the
-    property callers need who overlap launches on several streams.  The default mode refuses nothing but would stall
-    here, which is why the host never asks for such a grid."""
+def test_queue_survives_a_grid_the_device_cannot_hold(ds_weights):
+    """No workgroup owns an item before it runs, so even a grid of four times what the device holds at once
+    (workgroups that start only when others have left) finishes at once and correctly - the property callers need who
+    overlap launches on several streams.  Handing the first items out by workgroup index (ALPHA_MOE_STRICT_QUEUE=0, an
+    experiment switch) gives the same result on a grid the device holds."""
     import time
     P = make_problem(ds_weights, 16, seed=4)
     base = run_op(P, 16, 32, 8, 5, via="c_abi")
-    monkeypatch.setenv("ALPHA_MOE_STRICT_QUEUE", "1")
-    assert torch.equal(run_op(P, 16, 32, 8, 5, via="c_abi"), base)
-    monkeypatch.setenv("ALPHA_MOE_GRID", "1024")
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    got = run_op(P, 16, 32, 8, 5, via="c_abi")
-    dt = time.perf_counter() - t0
+    assert_parity(base, oracle_out(P), "ds M=16")
+    with tunables(ALPHA_MOE_STRICT_QUEUE=0):
+        assert torch.equal(run_op(P, 16, 32, 8, 5, via="c_abi"), base)
+    with tunables(ALPHA_MOE_GRID=1024):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        got = run_op(P, 16, 32, 8, 5, via="c_abi")
+        dt = time.perf_counter() - t0
     assert dt < 0.5, f"launch took {dt:.2f} s"
     assert torch.equal(got, base)
+    P = make_problem(ds_weights, 48, seed=4)   # whole-K UP items
+    base = run_op(P, 16, 32, 8, 5, via="c_abi")
+    with tunables(ALPHA_MOE_GRID=1024):
+        assert torch.equal(run_op(P, 16, 32, 8, 5, via="c_abi"), base)
 
 
-def test_strict_queue_two_streams_at_once(ds_weights, monkeypatch):
-    """Two launches in flight at the same time on two streams, each with a workspace of its own, in the mode made for
-    it: both finish at once and agree bit for bit with launches that ran alone."""
+def test_two_streams_at_once(ds_weights):
+    """Two launches in flight at the same time on two streams, each with a workspace of its own: both finish at once
+    and agree bit for bit with launches that ran alone."""
     import time
     import alpha_moe
-    monkeypatch.setenv("ALPHA_MOE_STRICT_QUEUE", "1")
     P1 = make_problem(ds_weights, 32, seed=5)
     P2 = make_problem(ds_weights, 24, seed=6)
     knobs = (16, 32, 8, 5)
@@ -501,3 +534,149 @@ def test_strict_queue_two_streams_at_once(ds_weights, monkeypatch):
     assert dt < 1.0, f"ten overlapping launches took {dt:.2f} s"
     for i, out in enumerate(outs):
         assert torch.equal(out, alone[i % 2]), i
+
+
+@pytest.mark.parametrize("name", ["ds", "qn"])
+def test_tiny_batches(name, ds_weights, qn_weights):
+    """M in {1, 2, 4, 8, 16}: K-split UP items whose partial sums the last arrival adds up (in batches of eight
+    splits), on both shards, several knobs, adding and storing, two launches bit for bit; against the oracle.  The 1e-2
+    bar holds on the benchmark sizes; on the sizes in between the bar is the random-shape test's (cosine >= 0.9999,
+    2e-2 of the range): with a dozen routed rows, one intermediate value that lands on the other side of an FP8
+    rounding boundary than the oracle's (its fp32 sums run in another order) moves a whole token by 1.2e-2 of the
+    range - seen at M=2."""
+    from oracle import moe_oracle as O
+    W = ds_weights if name == "ds" else qn_weights
+    benchmark_sizes = (1, 4, 16) if name == "ds" else (1,)
+    for M in (1, 2, 4, 8, 16):
+        P = make_problem(W, M, seed=20 + M)
+        ref = oracle_out(P)
+        for knobs in ((16, 32, 8, 5), (16, 64, 4, 3), (8, 32, 8, 2), (32, 64, 4, 4)):
+            print(f"case {name} M={M} knobs {knobs}", flush=True)
+            got = run_op(P, *knobs, via="c_abi")
+            if M in benchmark_sizes:
+                assert_parity(got, ref, f"{name} M={M} knobs {knobs}")
+            else:
+                m = O.error_metrics(got, ref)
+                assert m["cosine"] >= 0.9999 and m["max_abs_over_max_ref"] <= 2e-2, (name, M, knobs, m)
+            assert torch.equal(got, run_op(P, *knobs, via="c_abi")), (name, M, knobs)
+            junk = torch.full((P.M, P.shape.K), float("nan"), dtype=torch.bfloat16, device=DEV)
+            assert torch.equal(run_op(P, *knobs, out=junk, via="c_abi", store=True), got), (name, M, knobs, "store")
+        pre = torch.full((P.M, P.shape.K), 0.25, dtype=torch.bfloat16, device=DEV)
+        want = O.error_metrics(run_op(P, 16, 32, 8, 5, out=pre.clone(), via="c_abi"), oracle_out(P, out=pre.cpu()))
+        assert want["cosine"] >= 0.9999 and want["max_abs_over_max_ref"] <= 2e-2, (name, M, "out pre-filled", want)
+
+
+def test_tiny_batch_duplicates_padding_and_missing_experts():
+    """A tiny batch with what makes the bookkeeping interesting: a token that picks one expert twice (two rows of one
+    block), row blocks whose expert id is out of range (skipped), K % 256 == 128, three 128-column slices."""
+    shape = Shape("t", E=6, top_k=4, K=384, I=384, shared_expert=False, routing="softmax_renorm", scaling_factor=2.5,
+                  w_std=0.05)
+    W = make_weights(shape, device=DEV, seed=3)
+    P = make_problem(W, 12, seed=3)
+    g = torch.Generator(device=DEV).manual_seed(7)
+    P.topk_ids = torch.randint(0, 6, (12, 4), generator=g, device=DEV, dtype=torch.int32)   # with replacement
+    P.aligned.clear()
+    ref = oracle_out(P)
+    for knobs in ((8, 32, 8, 3), (16, 64, 4, 2), (32, 32, 8, 5)):
+        print(f"case tiny dup knobs {knobs}", flush=True)
+        got = run_op(P, *knobs, via="c_abi")
+        assert_parity(got, ref, f"tiny dup knobs {knobs}")
+        assert torch.equal(got, run_op(P, *knobs, via="c_abi"))
+    # experts 4 and 5 declared missing: their blocks are skipped, the others' results stay
+    s_ids, e_ids, total = P.align(16)
+    e_bad = torch.where(e_ids >= 4, torch.full_like(e_ids, -1), e_ids)
+    P.aligned[16] = (s_ids, e_bad, total)
+    keep = (P.topk_ids < 4)
+    saved = P.topk_weights
+    try:
+        print("case tiny missing experts", flush=True)
+        got = run_op(P, 16, 32, 8, 4, via="c_abi")
+        P.aligned.clear()
+        P.topk_weights = saved * keep   # the same thing said through the routing weights
+        want = oracle_out(P)
+    finally:
+        P.topk_weights = saved
+        P.aligned.clear()
+    assert_parity(got, want, "tiny missing experts")
+
+
+def test_ring_depth_is_clamped_to_what_lds_holds():
+    """block_m = 32 with stages = 5 and twelve 128-column slices asks for more LDS than a compute unit has next to the
+    item tables: the ring is made shallower instead of the launch failing."""
+    shape = Shape("wide", E=4, top_k=2, K=256, I=1536, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0,
+                  w_std=0.05)
+    W = make_weights(shape, device=DEV, seed=1)
+    P = make_problem(W, 40, seed=1)
+    ref = oracle_out(P)
+    for knobs in ((32, 64, 4, 5), (32, 32, 8, 5), (16, 64, 4, 5)):
+        print(f"case wide I=1536 knobs {knobs}", flush=True)
+        assert_parity(run_op(P, *knobs, via="c_abi"), ref, f"wide knobs {knobs}")
+
+
+def test_scratch_regrowth_after_graph_capture(c1):
+    """A graph captured on a stream keeps replaying into the scratch buffer the stream had then, also after a larger
+    eager call on the same stream made the binding take a bigger buffer; growth DURING capture is refused with an
+    error that names the remedy, and reserve_workspace makes the capture of the larger call possible."""
+    P, _ = c1
+    W = P.weights
+    knobs = (16, 32, 8, 3)
+    s_ids, e_ids, total = P.align(16)
+    out = torch.zeros((P.M, P.shape.K), dtype=torch.bfloat16, device=DEV)
+
+    def step(Q, ids, o, kn):
+        o.zero_()
+        torch.ops.alpha_moe.fused_moe_w8a8_up_down(Q.x, Q.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, *ids,
+                                                   Q.topk_weights, o, Q.shape.top_k, *kn, Q.shape.scaling_factor)
+
+    big = make_problem(W, 600, seed=8)
+    big_knobs = (128, 64, 4, 3)
+    big_ids = big.align(128)
+    big_out = torch.zeros((big.M, big.shape.K), dtype=torch.bfloat16, device=DEV)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(P, (s_ids, e_ids, total), out, knobs)
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step(P, (s_ids, e_ids, total), out, knobs)
+        # a larger call during another capture on this stream: refused, nothing recorded
+        g2 = torch.cuda.CUDAGraph()
+        with pytest.raises(RuntimeError, match="reserve_workspace"):
+            with torch.cuda.graph(g2, stream=side):
+                step(big, big_ids, big_out, big_knobs)
+        side.synchronize()
+        want = run_op(P, *knobs, via="c_abi")
+        graph.replay()
+        side.synchronize()
+        assert torch.equal(out, want)
+        # the larger call, eagerly, on the capture stream: the binding takes a bigger buffer ...
+        step(big, big_ids, big_out, big_knobs)
+        side.synchronize()
+        assert torch.equal(big_out, run_op(big, *big_knobs, via="c_abi"))
+        # ... and the graph still replays into the one it was captured with
+        for _ in range(3):
+            out.fill_(7.0)
+            graph.replay()
+            side.synchronize()
+            assert torch.equal(out, want)
+            step(big, big_ids, big_out, big_knobs)
+        side.synchronize()
+    # reserve first, then even the first call of a size may be captured
+    side2 = torch.cuda.Stream()
+    side2.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side2):
+        need = torch.ops.alpha_moe.workspace_bytes(big.shape.top_k, big.M, big.shape.K, big.shape.N, big.shape.E,
+                                                   big_ids[0].numel(), 128)
+        torch.ops.alpha_moe.reserve_workspace(big.x, need)
+        side2.synchronize()
+        g3 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g3, stream=side2):
+            step(big, big_ids, big_out, big_knobs)
+        big_out.fill_(3.0)
+        g3.replay()
+        side2.synchronize()
+        assert torch.equal(big_out, run_op(big, *big_knobs, via="c_abi"))
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.current_stream().wait_stream(side2)
+    torch.cuda.synchronize()
