@@ -181,6 +181,57 @@ extern "C" int alpha_moe_fused_moe_w8a8_up_down_store(const uint8_t *x, const fl
                          warp_n, stages, scaling_factor, workspace, workspace_bytes, stream, 1);
 }
 
+// ---- the entry point for callers that cannot allocate ------------------------------------------------------
+// Same call as alpha_moe_fused_moe_w8a8_up_down, with the scratch memory in this array instead of a caller's buffer.
+// Zero when the code object is loaded, which is the state the kernels' control prefix has to start in; afterwards the
+// kernels maintain it like any workspace.  Every device the library runs on holds its own copy until the process ends.
+static __device__ __align__(256) unsigned char scratch[ALPHA_MOE_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+// Device address of `scratch` on the current device: looked up once per device, with that device current (in host code
+// the array's name is a host-side handle, not a device address).
+void *static_scratch_of_current_device()
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static void *ptrs[kMaxDevices] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void *ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+        ptrs[dev] = ptr;
+    }
+    return ptrs[dev];
+}
+
+}  // namespace
+
+extern "C" int alpha_moe_fused_moe_w8a8_up_down_static(const uint8_t *x, const float *x_scale, const uint8_t *w,
+                                                       const float *w_scale, const uint8_t *w2, const float *w2_scale,
+                                                       uint16_t *out, const int32_t *sorted_token_ids,
+                                                       const int32_t *expert_ids,
+                                                       const int32_t *num_tokens_post_padded, const float *topk_weights,
+                                                       int top_k, int M, int K, int N, int num_experts, int sorted_num,
+                                                       int block_m, int block_n, int warp_n, int stages,
+                                                       float scaling_factor, void *stream)
+{
+    if (!x || !x_scale || !w || !w_scale || !w2 || !w2_scale || !out || !sorted_token_ids || !expert_ids ||
+        !num_tokens_post_padded || !topk_weights)
+        return ALPHA_MOE_ERR_NULL_POINTER;
+    const int rc = alpha_moe_validate(top_k, M, K, N, num_experts, sorted_num, block_m, block_n, warp_n, stages);
+    if (rc != ALPHA_MOE_OK) return rc;
+    if (alpha_moe_workspace_bytes(top_k, M, K, N, num_experts, sorted_num, block_m) > ALPHA_MOE_STATIC_SCRATCH_BYTES)
+        return ALPHA_MOE_ERR_SCRATCH_LIMIT;
+    void *ptr = static_scratch_of_current_device();
+    if (!ptr) return ALPHA_MOE_ERR_LAUNCH;
+    return run_fused_moe(x, x_scale, w, w_scale, w2, w2_scale, out, sorted_token_ids, expert_ids,
+                         num_tokens_post_padded, topk_weights, top_k, M, K, N, num_experts, sorted_num, block_m, block_n,
+                         warp_n, stages, scaling_factor, ptr, ALPHA_MOE_STATIC_SCRATCH_BYTES, stream, 0);
+}
+
 extern "C" int alpha_moe_workspace_check(const void *workspace, void *stream)
 {
     if (!workspace) return ALPHA_MOE_ERR_NULL_POINTER;
@@ -209,6 +260,9 @@ extern "C" const char *alpha_moe_status_string(int status)
     case ALPHA_MOE_ERR_WAIT_EXPIRED:
         return "a workgroup's bounded wait for another workgroup ran out in an earlier launch on this workspace: its "
                "results are not valid (launches overlapping on one device, or a device that cannot hold the grid)";
+    case ALPHA_MOE_ERR_SCRATCH_LIMIT:
+        return "the call needs more scratch memory than the library's built-in buffer holds "
+               "(alpha_moe_fused_moe_w8a8_up_down_static): use the entry point that takes a workspace";
     default: return "unknown status";
     }
 }

@@ -24,7 +24,8 @@ enum alpha_moe_status {
     ALPHA_MOE_ERR_STAGES = 5,         /* stages not in 1..5 */
     ALPHA_MOE_ERR_LAUNCH = 6,         /* the HIP runtime refused the launch (see hipGetLastError) */
     ALPHA_MOE_ERR_WORKSPACE = 7,      /* workspace null, misaligned or smaller than alpha_moe_workspace_bytes() */
-    ALPHA_MOE_ERR_WAIT_EXPIRED = 8    /* alpha_moe_workspace_check: a bounded wait between workgroups ran out */
+    ALPHA_MOE_ERR_WAIT_EXPIRED = 8,   /* alpha_moe_workspace_check: a bounded wait between workgroups ran out */
+    ALPHA_MOE_ERR_SCRATCH_LIMIT = 9   /* ..._static: the call needs more than ALPHA_MOE_STATIC_SCRATCH_BYTES of scratch */
 };
 
 /*
@@ -86,6 +87,31 @@ int alpha_moe_fused_moe_w8a8_up_down_store(
     int top_k, int M, int K, int N, int num_experts, int sorted_num,
     int block_m, int block_n, int warp_n, int stages,
     float scaling_factor, void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
+
+/*
+ * The adding call for callers that cannot allocate device memory or pass a buffer through: code under HIP graph
+ * capture that has no workspace at hand, tight serving loops, harnesses that forbid hipMalloc.  It has NO counterpart
+ * in the reference (whose kernel needs no scratch).  Same arguments, checks and result as
+ * alpha_moe_fused_moe_w8a8_up_down without `workspace` / `workspace_bytes`: the scratch memory is a buffer of
+ * ALPHA_MOE_STATIC_SCRATCH_BYTES built into the library's code object (every device the library runs on holds its own
+ * copy until the process ends).  The call allocates and frees nothing.  A call whose alpha_moe_workspace_bytes()
+ * exceeds that size returns ALPHA_MOE_ERR_SCRATCH_LIMIT and launches nothing: 64 MiB cover every decode-sized batch of
+ * the shipped shard shapes (DeepSeek-V3 shard: M <= 64) but not prefill.  All calls on one device share the one
+ * buffer, which keeps the last call's contents: calls that overlap in time on one device race (order them on one
+ * stream), and a bounded wait that ran out stays recorded for the life of the process (every later call then fills
+ * `out` with NaN).  The first call on a device looks the buffer's address up; make that call outside graph capture.
+ */
+#define ALPHA_MOE_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
+int alpha_moe_fused_moe_w8a8_up_down_static(
+    const uint8_t *x, const float *x_scale,
+    const uint8_t *w, const float *w_scale,
+    const uint8_t *w2, const float *w2_scale,
+    uint16_t *out,
+    const int32_t *sorted_token_ids, const int32_t *expert_ids, const int32_t *num_tokens_post_padded,
+    const float *topk_weights,
+    int top_k, int M, int K, int N, int num_experts, int sorted_num,
+    int block_m, int block_n, int warp_n, int stages,
+    float scaling_factor, void *stream /* hipStream_t */);
 
 /* Bytes of scratch the calls above need for these sizes (0 if any is not positive). */
 size_t alpha_moe_workspace_bytes(int top_k, int M, int K, int N, int num_experts, int sorted_num, int block_m);
