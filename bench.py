@@ -80,6 +80,7 @@ def main():
     n_routings = 8
 
     flush_buf = torch.empty((512 << 20) // 4, dtype=torch.int32, device=dev)
+    deferred_parity = []   # (result row, check) pairs run once every size has been timed
 
     def flush_caches(i):
         flush_buf.fill_(i)   # 512 MiB written: nothing of an earlier call is left in L2 or the Infinity Cache
@@ -124,12 +125,12 @@ def main():
             self.last = (P, W, s_ids, e_ids, total, out, knobs)
             return calls, statistics.mean(byts), statistics.mean(flops), knobs, src
 
-        def parity_sample(self, n=12):
+        def parity_sample(self, ctx, n=12):
             """The last prepared problem's output rows for a sample of its tokens against the CPU oracle on those tokens
             alone (a token's result depends only on its own row, routing and the weights)."""
             from oracle import moe_oracle as O
             from alpha_moe_python.workloads import Problem
-            P, W, s_ids, e_ids, total, out, knobs = self.last
+            P, W, s_ids, e_ids, total, out, knobs = ctx
             s = self.shape
             out.zero_()
             torch.ops.alpha_moe.fused_moe_w8a8_up_down(
@@ -158,8 +159,15 @@ def main():
             calls, B, F, knobs, src = self.prepare(M)
             # does the rotation alone keep a step's weights out of the 256 MiB Infinity Cache?
             cold = B * len(calls) < (1 << 30)
-            for i in range(warmup):
+            # W untimed steps, and at least 30 ms of them: the sizes are measured back to back with host work in
+            # between (building problems, the CPU oracle), and a GPU that has idled needs that long to clock up again
+            t_w = time.perf_counter()
+            i = 0
+            while i < warmup or time.perf_counter() - t_w < 0.03:
                 calls[i % len(calls)]()
+                i += 1
+                if i % 8 == 0:
+                    torch.cuda.synchronize()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             for i in range(steps):
@@ -180,8 +188,16 @@ def main():
                  "launch_us_median": statistics.median(dev_ms) * 1e3, "launch_us_min": min(dev_ms) * 1e3,
                  "bytes": B, "flops": F, "knobs": knobs, "knobs_from": src, "cold": cold}
             if not args.no_parity_samples:
-                r["parity_sample"] = self.parity_sample()
+                # checked after ALL timing is done: the CPU oracle takes a while, and a GPU that has idled meanwhile
+                # runs the next size's short measurement at lower clocks
+                ctx = self.last
+                deferred_parity.append((r, lambda ctx=ctx: self.parity_sample(ctx)))
             return r
+
+    def run_deferred_parity():
+        for r, check in deferred_parity:
+            r["summary"]["parity_sample"] = check()
+        deferred_parity.clear()
 
     def summarise(r):
         t_us = r["launch_us_mean"]
@@ -190,14 +206,13 @@ def main():
         extra = {"cold": r["cold"]}
         if r["cold"]:
             extra["us_per_layer_rotation_only"] = round(r["ms_per_step"] * 1e3, 2)
-        if "parity_sample" in r:
-            extra["parity_sample"] = r["parity_sample"]
-        return {"us_per_layer": round(us_layer, 2), "launch_us_mean": round(t_us, 2), **extra,
+        r["summary"] = {"us_per_layer": round(us_layer, 2), "launch_us_mean": round(t_us, 2), **extra,
                 "launch_us_median": round(r["launch_us_median"], 2),
                 "algorithmic_MB": round(r["bytes"] / 1e6, 1), "GB_per_s": round(r["bytes"] / t_us / 1e3, 1),
                 "hbm_frac": round(r["bytes"] / t_us / 1e3 / HBM_PEAK_GBS, 4),
                 "TFLOP_per_s": round(r["flops"] / t_us / 1e6, 2),
                 "mfma_frac": round(r["flops"] / t_us / 1e6 / FP8_PEAK_TFLOPS, 5), "knobs": r["knobs"]}
+        return r["summary"]
 
     def steps_for(M):
         return max(10, min(args.steps, args.steps * 64 // max(M, 64) * 2))
@@ -289,6 +304,7 @@ def main():
         result["parity"] = O.error_metrics(out, ref)
         del Wc
 
+    run_deferred_parity()
     if not args.no_other_configs and args.shape == "ds":
         del bench
         torch.cuda.empty_cache()
@@ -297,6 +313,7 @@ def main():
             b = Bench(name)
             other[name] = {"shape": f"E={b.shape.E} top_k={b.shape.top_k} K={b.shape.K} I={b.shape.I}",
                            "per_M": {str(m): summarise(b.measure(m, steps_for(m), min(args.warmup, 5))) for m in Ms}}
+            run_deferred_parity()
             del b
             torch.cuda.empty_cache()
         result["other_configs"] = other
