@@ -34,6 +34,10 @@ c_abi.alpha_moe_fused_moe_w8a8_up_down_store.argtypes = c_abi.alpha_moe_fused_mo
 c_abi.alpha_moe_fused_moe_w8a8_up_down_static.restype = ctypes.c_int
 c_abi.alpha_moe_fused_moe_w8a8_up_down_static.argtypes = (
     [ctypes.c_void_p] * 11 + [ctypes.c_int] * 10 + [ctypes.c_float, ctypes.c_void_p])
+c_abi.alpha_moe_fused_moe_w8a8_up_down_prepacked.restype = ctypes.c_int
+c_abi.alpha_moe_fused_moe_w8a8_up_down_prepacked.argtypes = (
+    [ctypes.c_void_p] * 11 + [ctypes.c_int] * 10 + [ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
+                                                   ctypes.c_void_p])
 c_abi.alpha_moe_set_tunable.restype = ctypes.c_int
 c_abi.alpha_moe_set_tunable.argtypes = [ctypes.c_char_p, ctypes.c_int, ctypes.c_int]
 c_abi.alpha_moe_workspace_check.restype = ctypes.c_int

@@ -22,6 +22,13 @@ def _fused_moe_w8a8_up_down_store_fake(x, x_scale, w, w_scale, w2, w2_scale, sor
     return None
 
 
+@torch.library.register_fake("alpha_moe::fused_moe_w8a8_up_down_prepacked")
+def _fused_moe_w8a8_up_down_prepacked_fake(x, x_scale, w_packed, w_scale, w2_packed, w2_scale, sorted_token_ids,
+                                           expert_ids, num_tokens_post_padded, topk_weights, out, top_k, block_m,
+                                           block_n, warp_n, stages, scaling_factor, store):
+    return None
+
+
 @torch.library.register_fake("alpha_moe::per_token_group_quant_fp8")
 def _per_token_group_quant_fp8_fake(x, group_size):
     return (torch.empty_like(x, dtype=torch.float8_e4m3fn),
@@ -81,4 +88,17 @@ def fused_moe_w8a8_up_down_store(x, x_scale, w, w_scale, w2, w2_scale, sorted_to
     return out
 
 
-__all__ = ["fused_moe_w8a8_up_down", "fused_moe_w8a8_up_down_store"]
+def fused_moe_w8a8_up_down_prepacked(x, x_scale, w_packed, w_scale, w2_packed, w2_scale, sorted_token_ids, expert_ids,
+                                     num_tokens_post_padded, topk_weights, out, top_k, block_m, block_n, warp_n, stages,
+                                     scaling_factor, store: bool = False) -> torch.Tensor:
+    """The operator on weights re-laid-out once by ``alpha_moe_python.utils.prepack_weights`` (``w_packed``
+    ``[E, K/128, N, 128]``, ``w2_packed`` ``[E, I/128, K, 128]``); every other argument as in
+    ``fused_moe_w8a8_up_down``, ``store=True`` for the overwriting variant.  Bit for bit the result of the call on the
+    unpacked weights.  The reference has no such variant.  Returns ``out``."""
+    torch.ops.alpha_moe.fused_moe_w8a8_up_down_prepacked(
+        x, x_scale, w_packed, w_scale, w2_packed, w2_scale, sorted_token_ids, expert_ids, num_tokens_post_padded,
+        topk_weights, out, top_k, block_m, block_n, warp_n, stages, scaling_factor, store)
+    return out
+
+
+__all__ = ["fused_moe_w8a8_up_down", "fused_moe_w8a8_up_down_store", "fused_moe_w8a8_up_down_prepacked"]

@@ -114,7 +114,8 @@ int run_fused_moe(const uint8_t *x, const float *x_scale, const uint8_t *w, cons
                   const float *w2_scale, uint16_t *out, const int32_t *sorted_token_ids, const int32_t *expert_ids,
                   const int32_t *num_tokens_post_padded, const float *topk_weights, int top_k, int M, int K, int N,
                   int num_experts, int sorted_num, int block_m, int block_n, int warp_n, int stages,
-                  float scaling_factor, void *workspace, size_t workspace_bytes, void *stream, int overwrite)
+                  float scaling_factor, void *workspace, size_t workspace_bytes, void *stream, int overwrite,
+                  int prepacked = 0)
 {
     if (!x || !x_scale || !w || !w_scale || !w2 || !w2_scale || !out || !sorted_token_ids || !expert_ids ||
         !num_tokens_post_padded || !topk_weights)
@@ -134,6 +135,11 @@ int run_fused_moe(const uint8_t *x, const float *x_scale, const uint8_t *w, cons
     p.top_k = top_k; p.M = M; p.K = K; p.N = N; p.E = num_experts; p.sorted_num = sorted_num; p.block_m = block_m;
     p.scaling = scaling_factor;
     p.overwrite = overwrite;
+    const size_t I = (size_t)N / 2;
+    p.w_rs = prepacked ? 128 : (size_t)K;
+    p.w_ks = prepacked ? (size_t)N * 128 : 128;
+    p.w2_rs = prepacked ? 128 : I;
+    p.w2_ks = prepacked ? (size_t)K * 128 : 128;
 
     hipStream_t hs = static_cast<hipStream_t>(stream);
     hipError_t err;
@@ -143,6 +149,8 @@ int run_fused_moe(const uint8_t *x, const float *x_scale, const uint8_t *w, cons
     } else if (path == kTile) {
         err = launch_tile(p, workspace, hs);
     } else {
+        // the fallback kernel reads the operator's own layout only
+        if (prepacked) return ALPHA_MOE_ERR_SHAPE;
         err = launch_zero_acc(p, hs);
         if (err == hipSuccess) err = launch_direct(p, warp_n, stages, hs);
         if (err == hipSuccess) err = launch_finalize(p, hs);
@@ -179,6 +187,21 @@ extern "C" int alpha_moe_fused_moe_w8a8_up_down_store(const uint8_t *x, const fl
     return run_fused_moe(x, x_scale, w, w_scale, w2, w2_scale, out, sorted_token_ids, expert_ids,
                          num_tokens_post_padded, topk_weights, top_k, M, K, N, num_experts, sorted_num, block_m, block_n,
                          warp_n, stages, scaling_factor, workspace, workspace_bytes, stream, 1);
+}
+
+extern "C" int alpha_moe_fused_moe_w8a8_up_down_prepacked(const uint8_t *x, const float *x_scale, const uint8_t *w_packed,
+                                                          const float *w_scale, const uint8_t *w2_packed,
+                                                          const float *w2_scale, uint16_t *out,
+                                                          const int32_t *sorted_token_ids, const int32_t *expert_ids,
+                                                          const int32_t *num_tokens_post_padded,
+                                                          const float *topk_weights, int top_k, int M, int K, int N,
+                                                          int num_experts, int sorted_num, int block_m, int block_n,
+                                                          int warp_n, int stages, float scaling_factor, int store,
+                                                          void *workspace, size_t workspace_bytes, void *stream)
+{
+    return run_fused_moe(x, x_scale, w_packed, w_scale, w2_packed, w2_scale, out, sorted_token_ids, expert_ids,
+                         num_tokens_post_padded, topk_weights, top_k, M, K, N, num_experts, sorted_num, block_m, block_n,
+                         warp_n, stages, scaling_factor, workspace, workspace_bytes, stream, store != 0, 1);
 }
 
 // ---- the entry point for callers that cannot allocate ------------------------------------------------------

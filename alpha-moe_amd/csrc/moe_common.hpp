@@ -44,6 +44,11 @@ struct MoeParams {
     int top_k, M, K, N, E, sorted_num, block_m;
     float scaling;
     int overwrite;              // 1: out = bf16(sum), whatever out held; 0: out = bf16(out + sum)
+    // Byte strides of the two weight tensors inside one expert: from one row to the next, and from one 128-byte K
+    // block of a row to the next.  The operator's layout ([N][K] and [K][I] row-major) has (K, 128) and (I, 128); the
+    // pre-packed layout ([K/128][N][128] and [I/128][K][128]: a K block of consecutive rows is contiguous) has
+    // (128, N * 128) and (128, K * 128).
+    size_t w_rs, w_ks, w2_rs, w2_ks;
 };
 
 __device__ __forceinline__ v4i ldg128(const uint8_t *p) { return *reinterpret_cast<const v4i *>(p); }

@@ -254,7 +254,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             for (int i = 0; i < 2; i++) {
                 // weight tile a = (pair a/2, gate|up a%2): tile row 8i + l/8 is slab row pair*32 + 16i + l/8 (+8 for up)
                 const int row = ib * 256 + wave * RW + (a >> 1) * 32 + 16 * i + ld_row + 8 * (a & 1);
-                ga[a][i] = p.w + ((size_t)e * p.N + row) * K + (size_t)kb0 * 128 + 16 * ld_chunk[i];
+                ga[a][i] = p.w + (size_t)e * p.N * K + row * p.w_rs + kb0 * p.w_ks + 16 * ld_chunk[i];
             }
         const uint8_t *gb[TM][2];
 #pragma unroll
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 if (a < TM)
                     dma16<0>(past_end ? dummy : gb[a < TM ? a : 0][i] + (size_t)kb * 128, dst + i * 1024);
                 else
-                    dma16<2>(past_end ? dummy : ga[a >= TM ? a - TM : 0][i] + (size_t)kb * 128, dst + i * 1024);
+                    dma16<2>(past_end ? dummy : ga[a >= TM ? a - TM : 0][i] + kb * p.w_ks, dst + i * 1024);
             }
         };
         int slot_w = 0, slot_r = 0;
@@ -408,15 +408,15 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             const uint8_t *gd[2];
 #pragma unroll
             for (int i = 0; i < 2; i++)
-                gd[i] = p.w2 + ((size_t)e * K + (size_t)(wng > 0 ? wt0 : 0) * 16 + 8 * i + ld_row) * I + 16 * ld_chunk[i];
-            const size_t group_step = (size_t)16 * I;
+                gd[i] = p.w2 + (size_t)e * K * I + ((wng > 0 ? wt0 : 0) * 16 + 8 * i + ld_row) * p.w2_rs + 16 * ld_chunk[i];
+            const size_t group_step = 16 * p.w2_rs;
             int ig = 0, iib = 0;   // (group, slice) of the next tile to issue
             auto issue = [&](int slot) {
                 uint8_t *dst = ring + slot * 2048;
                 const bool past_end = ig >= wng;
 #pragma unroll
                 for (int i = 0; i < 2; i++)
-                    dma16<2>(past_end ? dummy : gd[i] + ig * group_step + iib * 128, dst + i * 1024);
+                    dma16<2>(past_end ? dummy : gd[i] + ig * group_step + iib * p.w2_ks, dst + i * 1024);
                 iib++;
                 if (iib == n_ib) {
                     iib = 0;
@@ -508,15 +508,19 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     };
 
     auto fin_item = [&](int f) {
-        if (tid == 0) spin_until_ge(&s.ctl->down_done, n_down, s.ctl);
+        if (tid == 0) {
+            spin_until_ge(&s.ctl->down_done, n_down, s.ctl);
+            // A bounded wait that ran out - in this launch or in an earlier one on this workspace: the word is sticky -
+            // means that some result rows may be missing.  The output then says so itself: NaN in every element.
+            // One thread asks (agent-scope loads of one word from every wavefront queue up at the memory side).
+            s_bcast[1] = load_agent(&s.ctl->error);
+        }
         __syncthreads();
         const int t = f / s.n_fc;
         const int c = (f - t * s.n_fc) * kFinCols + tid * 4;
         // lane k fetches the stamp of the token's slot k: one round trip for all of them (top_k <= 64)
         const int stamp = load_agent(&s.live[t * p.top_k + (lane < p.top_k ? lane : 0)]);
-        // A bounded wait that ran out - in this launch or in an earlier one on this workspace: the word is sticky - means
-        // that some result rows may be missing.  The output then says so itself: NaN in every element.
-        const bool poisoned = load_agent(&s.ctl->error) != 0;
+        const bool poisoned = s_bcast[1] != 0;
         const unsigned long long live_mask = __ballot(lane < p.top_k && stamp == epoch);
         if (poisoned) {
             if (tid < kFinCols / 4 && c < K)

@@ -212,13 +212,13 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         // Weight rows of the pair: tile a = (32-row group a / 2, gate | up a % 2); matrix row r of the tile is slab row
         // group * 32 + (r / 8) * 16 + r % 8 (+ 8 for up), so load h of a tile covers slab rows ... + 16 h + lane / 8.
         // Wavefront (w, g) loads tiles 2g and 2g + 1 of pair w.
-        const uint8_t *wbase = p.w + ((size_t)e * p.N + ib * 256 + w * 64 + g * 32 + ld_row) * K;
+        const uint8_t *wbase = p.w + (size_t)e * p.N * K + (ib * 256 + w * 64 + g * 32 + ld_row) * p.w_rs;
         // operation i of a step's OPS1: weight tile half (i < AOPS), token tile half, token scales
         auto issue_op = [&](int kb, int stage, int i) {
             const int kc = kb < nkb ? kb : nkb - 1;
             if (i < AOPS) {
                 const int up = i >> 1, h = i & 1;
-                const uint8_t *src = wbase + (size_t)(h * 16 + 8 * up) * K + (size_t)kc * 128 + ld_chunk[h];
+                const uint8_t *src = wbase + (h * 16 + 8 * up) * p.w_rs + kc * p.w_ks + ld_chunk[h];
                 uint8_t *dst = a_ring + stage * 8192 + (2 * g + up) * 2048 + h * 1024;
                 if (nt) dma16<2>(src, dst);
                 else dma16<0>(src, dst);
@@ -339,7 +339,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         int my_groups = (span - w + 3) >> 2;                      // the slab's groups w, w + 4, ... (none: 0)
         my_groups = my_groups > 0 ? my_groups : 0;
         const int n_steps = ((span + 3) >> 2) * n_ib;             // (group, slice) steps of the longest pair, slice-minor
-        const uint8_t *w2base = p.w2 + ((size_t)e * K + 16 * (lane >> 5) + (ld_row & 3)) * I;
+        const uint8_t *w2base = p.w2 + (size_t)e * K * I + (16 * (lane >> 5) + (ld_row & 3)) * p.w2_rs;
         int lg = 0, lib = 0;   // (group index, slice) of the next step to load
         auto group_of = [&](int i) {   // i-th group of this pair, clamped into the slab for loads past its end
             int grp = g0 + w + 4 * (i < my_groups ? i : my_groups - 1);
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         auto issue2_op = [&](int stage, int i) {   // operation i of AOPS of the step (lg, lib)
             const int c0 = group_of(lg) << 6;
             const int k = 2 * g + (i >> 1), h = i & 1;
-            const uint8_t *src = w2base + (size_t)(c0 + 32 * h + 4 * k) * I + lib * 128 + ld_chunk[h];
+            const uint8_t *src = w2base + (c0 + 32 * h + 4 * k) * p.w2_rs + lib * p.w2_ks + ld_chunk[h];
             uint8_t *dst = a_ring + stage * 8192 + k * 2048 + h * 1024;
             if (nt) dma16<2>(src, dst);
             else dma16<0>(src, dst);
@@ -526,7 +526,9 @@ __global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams s
     const int epoch = (int)((unsigned)s.ctl->epoch + 1u);
     // a bounded wait that ran out (in this call's tile kernel or in any earlier launch on this workspace: the word is
     // sticky) means result rows may be missing: the output then says so itself, NaN in every element
-    const bool poisoned = load_agent(&s.ctl->error) != 0;
+    // (an ordinary load: this kernel starts after the tile kernel has ended, and every wavefront asking the memory side
+    // for the same word with an agent-scope load cost ~100 us per call)
+    const bool poisoned = s.ctl->error != 0;
     for (int unit = blockIdx.x; unit < n_units; unit += gridDim.x) {
         const int t = unit / chunks_per_token;
         const int c = (unit - t * chunks_per_token) * 2048 + threadIdx.x * 8;

@@ -92,7 +92,7 @@ void run_fused_moe(const at::Tensor &x, const at::Tensor &x_scale, const at::Ten
                    const at::Tensor &w2, const at::Tensor &w2_scale, const at::Tensor &sorted_token_ids,
                    const at::Tensor &expert_ids, const at::Tensor &num_tokens_post_padded,
                    const at::Tensor &topk_weights, at::Tensor &out, int64_t top_k, int64_t block_m, int64_t block_n,
-                   int64_t warp_n, int64_t stages, double scaling_factor, bool store)
+                   int64_t warp_n, int64_t stages, double scaling_factor, bool store, bool prepacked = false)
 {
     TORCH_CHECK(x.is_cuda(), "x must be a GPU tensor");
     const at::Device dev = x.device();
@@ -111,10 +111,20 @@ void run_fused_moe(const at::Tensor &x, const at::Tensor &x_scale, const at::Ten
     TORCH_CHECK(x.dim() == 2 && x.size(0) > 0, "x must be [M, K] with M > 0");
     const int64_t M = x.size(0), K = x.size(1);
     TORCH_CHECK(K % 128 == 0, "K dimension must be a multiple of 128");
-    TORCH_CHECK(w.dim() == 3 && w.size(2) == K, "w must be [E, N, K] with the K of x");
-    const int64_t E = w.size(0), N = w.size(1);
-    TORCH_CHECK(N % 256 == 0, "N (= 2 * intermediate size) must be a multiple of 256");
-    TORCH_CHECK(w2.dim() == 3 && w2.size(0) == E && w2.size(1) == K && w2.size(2) == N / 2, "w2 must be [E, K, N/2]");
+    int64_t E, N;
+    if (!prepacked) {
+        TORCH_CHECK(w.dim() == 3 && w.size(2) == K, "w must be [E, N, K] with the K of x");
+        E = w.size(0), N = w.size(1);
+        TORCH_CHECK(N % 256 == 0, "N (= 2 * intermediate size) must be a multiple of 256");
+        TORCH_CHECK(w2.dim() == 3 && w2.size(0) == E && w2.size(1) == K && w2.size(2) == N / 2, "w2 must be [E, K, N/2]");
+    } else {
+        TORCH_CHECK(w.dim() == 4 && w.size(1) == K / 128 && w.size(3) == 128,
+                    "w_packed must be [E, K/128, N, 128] with the K of x (alpha_moe_python.utils.prepack_weights)");
+        E = w.size(0), N = w.size(2);
+        TORCH_CHECK(N % 256 == 0, "N (= 2 * intermediate size) must be a multiple of 256");
+        TORCH_CHECK(w2.dim() == 4 && w2.size(0) == E && w2.size(1) == N / 256 && w2.size(2) == K && w2.size(3) == 128,
+                    "w2_packed must be [E, N/256, K, 128]");
+    }
     TORCH_CHECK(x_scale.numel() == M * (K / 128), "x_scale must be [M, K/128]");
     TORCH_CHECK(w_scale.numel() == E * (N / 128) * (K / 128), "w_scale must be [E, N/128, K/128]");
     TORCH_CHECK(w2_scale.numel() == E * (K / 128) * (N / 256), "w2_scale must be [E, K/128, N/256]");
@@ -139,18 +149,29 @@ void run_fused_moe(const at::Tensor &x, const at::Tensor &x_scale, const at::Ten
                                   static_cast<int>(E), static_cast<int>(sorted_num), static_cast<int>(block_m));
     at::Tensor ws = workspace_for(dev, stream, ws_bytes);
 
-    const auto entry = store ? alpha_moe_fused_moe_w8a8_up_down_store : alpha_moe_fused_moe_w8a8_up_down;
-    const int rc = entry(
-        static_cast<const uint8_t *>(x.const_data_ptr()), x_scale.const_data_ptr<float>(),
-        static_cast<const uint8_t *>(w.const_data_ptr()), w_scale.const_data_ptr<float>(),
-        static_cast<const uint8_t *>(w2.const_data_ptr()), w2_scale.const_data_ptr<float>(),
-        static_cast<uint16_t *>(out.data_ptr()), sorted_token_ids.const_data_ptr<int32_t>(),
-        expert_ids.const_data_ptr<int32_t>(), num_tokens_post_padded.const_data_ptr<int32_t>(),
-        topk_weights.const_data_ptr<float>(), static_cast<int>(top_k), static_cast<int>(M), static_cast<int>(K),
-        static_cast<int>(N), static_cast<int>(E), static_cast<int>(sorted_num), static_cast<int>(block_m),
-        static_cast<int>(block_n), static_cast<int>(warp_n), static_cast<int>(stages),
-        static_cast<float>(scaling_factor), ws.data_ptr(), static_cast<size_t>(ws.numel()),
-        static_cast<void *>(stream));
+    const int rc = (prepacked ?
+        alpha_moe_fused_moe_w8a8_up_down_prepacked(
+            static_cast<const uint8_t *>(x.const_data_ptr()), x_scale.const_data_ptr<float>(),
+            static_cast<const uint8_t *>(w.const_data_ptr()), w_scale.const_data_ptr<float>(),
+            static_cast<const uint8_t *>(w2.const_data_ptr()), w2_scale.const_data_ptr<float>(),
+            static_cast<uint16_t *>(out.data_ptr()), sorted_token_ids.const_data_ptr<int32_t>(),
+            expert_ids.const_data_ptr<int32_t>(), num_tokens_post_padded.const_data_ptr<int32_t>(),
+            topk_weights.const_data_ptr<float>(), static_cast<int>(top_k), static_cast<int>(M), static_cast<int>(K),
+            static_cast<int>(N), static_cast<int>(E), static_cast<int>(sorted_num), static_cast<int>(block_m),
+            static_cast<int>(block_n), static_cast<int>(warp_n), static_cast<int>(stages),
+            static_cast<float>(scaling_factor), store ? 1 : 0, ws.data_ptr(), static_cast<size_t>(ws.numel()),
+            static_cast<void *>(stream))
+        : (store ? alpha_moe_fused_moe_w8a8_up_down_store : alpha_moe_fused_moe_w8a8_up_down)(
+            static_cast<const uint8_t *>(x.const_data_ptr()), x_scale.const_data_ptr<float>(),
+            static_cast<const uint8_t *>(w.const_data_ptr()), w_scale.const_data_ptr<float>(),
+            static_cast<const uint8_t *>(w2.const_data_ptr()), w2_scale.const_data_ptr<float>(),
+            static_cast<uint16_t *>(out.data_ptr()), sorted_token_ids.const_data_ptr<int32_t>(),
+            expert_ids.const_data_ptr<int32_t>(), num_tokens_post_padded.const_data_ptr<int32_t>(),
+            topk_weights.const_data_ptr<float>(), static_cast<int>(top_k), static_cast<int>(M), static_cast<int>(K),
+            static_cast<int>(N), static_cast<int>(E), static_cast<int>(sorted_num), static_cast<int>(block_m),
+            static_cast<int>(block_n), static_cast<int>(warp_n), static_cast<int>(stages),
+            static_cast<float>(scaling_factor), ws.data_ptr(), static_cast<size_t>(ws.numel()),
+            static_cast<void *>(stream)));
     TORCH_CHECK(rc == ALPHA_MOE_OK, "alpha_moe_fused_moe_w8a8_up_down failed: ", alpha_moe_status_string(rc));
 }
 
@@ -175,6 +196,20 @@ void fused_moe_w8a8_up_down_store(const at::Tensor &x, const at::Tensor &x_scale
 {
     run_fused_moe(x, x_scale, w, w_scale, w2, w2_scale, sorted_token_ids, expert_ids, num_tokens_post_padded,
                   topk_weights, out, top_k, block_m, block_n, warp_n, stages, scaling_factor, true);
+}
+
+// The operator on weights re-laid-out by alpha_moe_python.utils.prepack_weights: w_packed [E, K/128, N, 128],
+// w2_packed [E, I/128, K, 128]; store selects the overwriting variant.
+void fused_moe_w8a8_up_down_prepacked(const at::Tensor &x, const at::Tensor &x_scale, const at::Tensor &w_packed,
+                                      const at::Tensor &w_scale, const at::Tensor &w2_packed, const at::Tensor &w2_scale,
+                                      const at::Tensor &sorted_token_ids, const at::Tensor &expert_ids,
+                                      const at::Tensor &num_tokens_post_padded, const at::Tensor &topk_weights,
+                                      at::Tensor &out, int64_t top_k, int64_t block_m, int64_t block_n, int64_t warp_n,
+                                      int64_t stages, double scaling_factor, bool store)
+{
+    run_fused_moe(x, x_scale, w_packed, w_scale, w2_packed, w2_scale, sorted_token_ids, expert_ids,
+                  num_tokens_post_padded, topk_weights, out, top_k, block_m, block_n, warp_n, stages, scaling_factor, store,
+                  true);
 }
 
 // (q, scale) = per_token_group_quant_fp8(x, 128): what the reference's callers get from SGLang (jit_moe.py:142).
@@ -250,4 +285,10 @@ TORCH_LIBRARY_FRAGMENT(alpha_moe, m)
           "Tensor(a!) out, int top_k, int block_m, int block_n, int warp_n, int stages, float scaling_factor"
           ") -> ()");
     m.impl("fused_moe_w8a8_up_down_store", c10::DispatchKey::CUDA, &fused_moe_w8a8_up_down_store);
+    m.def("fused_moe_w8a8_up_down_prepacked("
+          "Tensor x, Tensor x_scale, Tensor w_packed, Tensor w_scale, Tensor w2_packed, Tensor w2_scale, "
+          "Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_post_padded, Tensor topk_weights, "
+          "Tensor(a!) out, int top_k, int block_m, int block_n, int warp_n, int stages, float scaling_factor, bool store"
+          ") -> ()");
+    m.impl("fused_moe_w8a8_up_down_prepacked", c10::DispatchKey::CUDA, &fused_moe_w8a8_up_down_prepacked);
 }

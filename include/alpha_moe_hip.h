@@ -89,6 +89,29 @@ int alpha_moe_fused_moe_w8a8_up_down_store(
     float scaling_factor, void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
 
 /*
+ * The same operator on PRE-PACKED weights (an optional offline re-layout; the interleave-8 layout above stays the
+ * operator's API).  No counterpart in the reference, whose TMA box loads take the row-major tensors as they are; it
+ * builds on the reference's interleave step (alpha_moe_python/utils.py:5-17, README.md:94-102) and is applied after it:
+ *   w_packed   [E, K/128, N, 128]  = w  viewed as [E, N, K/128, 128] with the two middle axes swapped
+ *   w2_packed  [E, I/128, K, 128]  = w2 viewed as [E, K, I/128, 128] with the two middle axes swapped
+ * so that one 128-byte K block of consecutive rows is contiguous in memory: the 256 rows of a slice are one 32 KiB
+ * burst per K step instead of 256 row pieces K bytes apart.  alpha_moe_python.utils.prepack_weights builds both.
+ * Scales, routing arrays, knobs, workspace and status codes are those of alpha_moe_fused_moe_w8a8_up_down; store != 0
+ * gives the semantics of ..._store.  Shapes that only the fallback kernel takes (more than eight 128-column slices, K
+ * above 16384) return ALPHA_MOE_ERR_SHAPE: that kernel reads the operator's layout only.
+ */
+int alpha_moe_fused_moe_w8a8_up_down_prepacked(
+    const uint8_t *x, const float *x_scale,
+    const uint8_t *w_packed, const float *w_scale,
+    const uint8_t *w2_packed, const float *w2_scale,
+    uint16_t *out,
+    const int32_t *sorted_token_ids, const int32_t *expert_ids, const int32_t *num_tokens_post_padded,
+    const float *topk_weights,
+    int top_k, int M, int K, int N, int num_experts, int sorted_num,
+    int block_m, int block_n, int warp_n, int stages,
+    float scaling_factor, int store, void *workspace, size_t workspace_bytes, void *stream /* hipStream_t */);
+
+/*
  * The adding call for callers that cannot allocate device memory or pass a buffer through: code under HIP graph
  * capture that has no workspace at hand, tight serving loops, harnesses that forbid hipMalloc.  It has NO counterpart
  * in the reference (whose kernel needs no scratch).  Same arguments, checks and result as

@@ -680,3 +680,60 @@ def test_scratch_regrowth_after_graph_capture(c1):
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.current_stream().wait_stream(side2)
     torch.cuda.synchronize()
+
+
+def _run_prepacked(P, packed, knobs, store=False, via="c_abi", out=None):
+    import alpha_moe
+    wp, w2p = packed
+    W = P.weights
+    s_ids, e_ids, total = P.align(knobs[0])
+    if out is None:
+        out = torch.zeros((P.M, P.shape.K), dtype=torch.bfloat16, device=DEV)
+    if via == "torch":
+        torch.ops.alpha_moe.fused_moe_w8a8_up_down_prepacked(P.x, P.x_scale, wp, W.w1_scale, w2p, W.w2_scale, s_ids, e_ids,
+                                                             total, P.topk_weights, out, P.shape.top_k, *knobs,
+                                                             P.shape.scaling_factor, store)
+    else:
+        need = alpha_moe.c_abi.alpha_moe_workspace_bytes(P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E, s_ids.numel(), knobs[0])
+        ws = torch.zeros(need, dtype=torch.uint8, device=DEV)
+        rc = alpha_moe.c_abi.alpha_moe_fused_moe_w8a8_up_down_prepacked(
+            P.x.data_ptr(), P.x_scale.data_ptr(), wp.data_ptr(), W.w1_scale.data_ptr(), w2p.data_ptr(),
+            W.w2_scale.data_ptr(), out.data_ptr(), s_ids.data_ptr(), e_ids.data_ptr(), total.data_ptr(),
+            P.topk_weights.data_ptr(), P.shape.top_k, P.M, P.shape.K, P.shape.N, P.shape.E, s_ids.numel(), *knobs,
+            float(P.shape.scaling_factor), 1 if store else 0, ws.data_ptr(), ws.numel(),
+            torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, alpha_moe.c_abi.alpha_moe_status_string(rc)
+    torch.cuda.synchronize()
+    return out
+
+
+def test_prepacked_weights_give_the_same_bits(c1, ds_weights, q3_weights):
+    """fused_moe_w8a8_up_down_prepacked on prepack_weights(w, w2) against the operator on w, w2: bit for bit, streaming
+    and tile kernels, adding and storing, torch op and C ABI - on the CPU-sized case, the DeepSeek-V3 shard at M=256 and
+    the Zipf shard at M=200 (six slices)."""
+    from alpha_moe_python.utils import prepack_weights
+    P, ref = c1
+    packed = prepack_weights(P.weights.w1, P.weights.w2)
+    for knobs in ((16, 32, 8, 5), (16, 64, 4, 2), (32, 64, 4, 3), (64, 64, 4, 3), (128, 64, 4, 3)):
+        print(f"case prepacked c1 knobs {knobs}", flush=True)
+        want = run_op(P, *knobs, via="c_abi")
+        for via in ("c_abi", "torch"):
+            assert torch.equal(_run_prepacked(P, packed, knobs, via=via), want), (knobs, via)
+        junk = torch.full((P.M, P.shape.K), float("nan"), dtype=torch.bfloat16, device=DEV)
+        assert torch.equal(_run_prepacked(P, packed, knobs, store=True, out=junk), want), (knobs, "store")
+    assert_parity(_run_prepacked(P, packed, (16, 32, 8, 5)), ref, "prepacked c1")
+    for W, M, knob_list in ((ds_weights, 256, ((16, 64, 4, 3), (64, 64, 4, 3), (128, 64, 4, 3))),
+                            (q3_weights, 200, ((16, 32, 8, 5), (64, 64, 4, 3), (128, 64, 4, 2)))):
+        Q = make_problem(W, M, seed=1)
+        packed = prepack_weights(W.w1, W.w2)
+        for knobs in knob_list:
+            print(f"case prepacked {W.shape.name} M={M} knobs {knobs}", flush=True)
+            assert torch.equal(_run_prepacked(Q, packed, knobs), run_op(Q, *knobs, via="c_abi")), (W.shape.name, knobs)
+        del packed
+    # shapes only the fallback kernel takes are refused for pre-packed weights
+    import alpha_moe
+    shape = Shape("fb", E=2, top_k=1, K=128, I=1152, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0)
+    Wf = make_weights(shape, device=DEV, seed=5)
+    Pf = make_problem(Wf, 8, seed=5)
+    with pytest.raises(AssertionError):
+        _run_prepacked(Pf, prepack_weights(Wf.w1, Wf.w2), (128, 64, 4, 2))

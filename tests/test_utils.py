@@ -77,3 +77,32 @@ def test_get_best_config_on_reference_tables(tmp_path):
     for cfg in ds["entries"].values():
         assert set(cfg) == {"block_m", "block_n", "warp_n", "stages"}
         assert cfg["block_n"] * cfg["warp_n"] == 256
+
+
+def test_prepack_weights_is_the_stated_permutation_and_round_trips():
+    """w_packed[e, kb, n, :] = w[e, n, 128 kb : 128 kb + 128] and w2_packed[e, ib, c, :] = w2[e, c, 128 ib : 128 ib + 128]
+    (brute force over every index of a small case), any dtype, and unpack_weights is the inverse."""
+    import torch
+    from alpha_moe_python.utils import prepack_weights, unpack_weights
+    E, N, K = 3, 512, 384
+    w = torch.arange(E * N * K, dtype=torch.int32).reshape(E, N, K)
+    w2 = torch.arange(E * K * (N // 2), dtype=torch.int32).reshape(E, K, N // 2) + 7
+    wp, w2p = prepack_weights(w, w2)
+    assert tuple(wp.shape) == (E, K // 128, N, 128) and tuple(w2p.shape) == (E, N // 256, K, 128)
+    assert wp.is_contiguous() and w2p.is_contiguous()
+    for e in range(E):
+        for kb in range(K // 128):
+            for n in (0, 1, 7, 8, 255, 256, N - 1):
+                assert torch.equal(wp[e, kb, n], w[e, n, 128 * kb:128 * kb + 128])
+        for ib in range(N // 256):
+            for c in (0, 5, 127, 128, K - 1):
+                assert torch.equal(w2p[e, ib, c], w2[e, c, 128 * ib:128 * ib + 128])
+    back = unpack_weights(wp, w2p)
+    assert torch.equal(back[0], w) and torch.equal(back[1], w2)
+    q = torch.randn(2, 256, 128).to(torch.float8_e4m3fn)
+    q2 = torch.randn(2, 128, 128).to(torch.float8_e4m3fn)
+    a, b = prepack_weights(q, q2)
+    assert a.dtype == torch.float8_e4m3fn and torch.equal(unpack_weights(a, b)[0].view(torch.uint8), q.view(torch.uint8))
+    import pytest
+    with pytest.raises(ValueError):
+        prepack_weights(torch.zeros(2, 256, 100), torch.zeros(2, 100, 128))
