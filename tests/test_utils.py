@@ -106,3 +106,27 @@ def test_prepack_weights_is_the_stated_permutation_and_round_trips():
     import pytest
     with pytest.raises(ValueError):
         prepack_weights(torch.zeros(2, 256, 100), torch.zeros(2, 100, 128))
+
+
+def test_sglang_weight_loader_bookkeeping():
+    import torch
+    from alpha_moe_python.sglang_glue import W13Interleaver
+    from alpha_moe_python.utils import interleave_tensor
+    """Shards may arrive in any order, as w1 + w3 or as one fused w13; the slot is interleaved exactly once, when
+    complete, and other shard ids are ignored."""
+    E, I, K = 3, 16, 8
+    ckpt = torch.arange(E * 2 * I * K, dtype=torch.float32).reshape(E, 2 * I, K)
+    param = torch.zeros_like(ckpt)
+    il = W13Interleaver(E, rep=8)
+    order = [(0, "w3"), (1, "w1"), (0, "w2"), (0, "w1"), (2, "w13"), (1, "w3")]
+    done = []
+    for e, shard in order:
+        if shard == "w1":
+            param[e, :I] = ckpt[e, :I]
+        elif shard == "w3":
+            param[e, I:] = ckpt[e, I:]
+        elif shard == "w13":
+            param[e] = ckpt[e]
+        done.append(il.shard_loaded(param[e], e, shard))
+    assert done == [False, False, False, True, True, True]
+    assert torch.equal(param, interleave_tensor(ckpt, 8))
