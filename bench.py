@@ -30,9 +30,11 @@ sys.path.insert(0, os.path.join(ROOT, "alpha-moe_amd"))
 sys.path.insert(0, ROOT)
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy of known size), for the
-# configurations that were profiled: profiles/moe_stream_kernel_ds_decode_M64_hbm_traffic.md
-#   profiles/moe_tile_kernel_ds_prefill_M8192_hbm_traffic.md (both kernels of a call)
-MEASURED_TRAFFIC_BYTES = {("ds", 64): 1294.9e6, ("ds", 8192): 4812.2e6}
+# configurations that were profiled (all kernels of a call):
+#   profiles/moe_stream_kernel_ds_decode_M64_hbm_traffic.md, profiles/moe_tile_kernel_ds_prefill_M8192_hbm_traffic.md,
+#   profiles/moe_tile_kernel_q3_prefill_M8192_hbm_traffic.md
+MEASURED_TRAFFIC_BYTES = {("ds", 64): 1293.9e6, ("ds", 512): 1676.0e6, ("ds", 2048): 2240.8e6, ("ds", 8192): 4802.9e6,
+                          ("q3", 1024): 813.4e6, ("q3", 8192): 1897.0e6}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
 DEFAULT_KNOBS = {"block_m": 16, "block_n": 32, "warp_n": 8, "stages": 5}
@@ -184,7 +186,7 @@ def main():
                 evs[i][1].record()
             torch.cuda.synchronize()
             dev_ms = [a.elapsed_time(b) for a, b in evs]
-            r = {"M": M, "ms_per_step": wall_ms, "launch_us_mean": statistics.mean(dev_ms) * 1e3,
+            r = {"M": M, "shape": self.shape.name, "ms_per_step": wall_ms, "launch_us_mean": statistics.mean(dev_ms) * 1e3,
                  "launch_us_median": statistics.median(dev_ms) * 1e3, "launch_us_min": min(dev_ms) * 1e3,
                  "bytes": B, "flops": F, "knobs": knobs, "knobs_from": src, "cold": cold}
             if not args.no_parity_samples:
@@ -206,6 +208,8 @@ def main():
         extra = {"cold": r["cold"]}
         if r["cold"]:
             extra["us_per_layer_rotation_only"] = round(r["ms_per_step"] * 1e3, 2)
+        if (r["shape"], r["M"]) in MEASURED_TRAFFIC_BYTES:
+            extra["traffic_MB"] = round(MEASURED_TRAFFIC_BYTES[(r["shape"], r["M"])] / 1e6, 1)
         r["summary"] = {"us_per_layer": round(us_layer, 2), "launch_us_mean": round(t_us, 2), **extra,
                 "launch_us_median": round(r["launch_us_median"], 2),
                 "algorithmic_MB": round(r["bytes"] / 1e6, 1), "GB_per_s": round(r["bytes"] / t_us / 1e3, 1),
