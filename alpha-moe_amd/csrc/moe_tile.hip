@@ -48,6 +48,24 @@ constexpr int kStages = 3;
 constexpr int kARingBytes = 4 * kStages * 8192;   // 4 wavefronts x 3 stages x 4 tiles of 2 KiB
 constexpr int kMaxTailBytes = 48 << 10;           // token-tile ring / requantised tiles next to the weight rings
 
+// Measurement builds only (-DALPHA_MOE_TILE_PROBE=<bits>, microbench/tile_phase_probe.py): parts of the kernel are
+// compiled out to time the rest.  Results are then wrong on purpose.  The library is built without the macro, and
+// every TILE_PROBE() below is then a constant false.
+enum : int {
+    kProbeNoUp = 1,       // up/gate items only stamp their flag
+    kProbeNoDown = 2,     // down items are skipped
+    kProbeNoY = 4,        // down items do not store their result rows
+    kProbeNoReduce = 8,   // the reduce kernel is not launched
+    kProbeRow0 = 16,      // every routed row gathers token 0 (token tiles come from L2)
+    kProbeExpert8 = 32,   // expert e reads the weights of expert e % 8 (weights come from L2 / Infinity Cache)
+    kProbeNoLoad = 64,    // up/gate items issue no loads (matrix work on whatever LDS holds)
+    kProbeNoMma = 128,    // steps issue their loads and do no matrix or vector work
+};
+#ifndef ALPHA_MOE_TILE_PROBE
+#define ALPHA_MOE_TILE_PROBE 0
+#endif
+#define TILE_PROBE(bits) (((ALPHA_MOE_TILE_PROBE) & (bits)) != 0)
+
 struct TileParams {
     MoeParams p;
     StreamCtl *ctl;
@@ -70,9 +88,15 @@ struct TileParams {
 // load instruction blocks its wavefront for 30-60 ns (measured), and the other wavefront of the SIMD computes then.
 template <int TH, int NOPS, typename Issue>
 __device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *b_tiles, const float *row, float sc0,
-                                         float sc1, v4f (&acc)[4][TH], int frag_lo, int frag_hi, Issue issue)
+                                         float sc1, v4f (&acc)[4][TH], int frag_lo, int frag_hi, Issue issue,
+                                         bool loads_only = false)
 {
     constexpr int GROUPS = 4 * TH;
+    if (loads_only) {   // constant false outside measurement builds
+#pragma unroll
+        for (int i = 0; i < NOPS; i++) issue(i);
+        return;
+    }
     auto read_tile = [&](const uint8_t *tile) -> v8i {
         return cat(*reinterpret_cast<const v4i *>(tile + frag_lo), *reinterpret_cast<const v4i *>(tile + frag_hi));
     };
@@ -185,15 +209,16 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
     };
 
     auto up_item = [&](int mb, int ib) {
-        const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
+        int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
         if (e < 0 || e >= p.E) return;
+        if (TILE_PROBE(kProbeExpert8)) e &= 7;
         const bool nt = lone_block(mb, e);
         if (tid < TM * 16) {
             const int idx = mb * p.block_m + tid;
             int id = -1;
             if (tid < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
             const int tk = id / p.top_k;
-            s_tok[tid] = (id >= 0 && tk < p.M) ? tk : 0;
+            s_tok[tid] = (id >= 0 && tk < p.M && !TILE_PROBE(kProbeRow0)) ? tk : 0;
         }
         // this slice's gate (row 2*ib) and up (row 2*ib+1) scale rows
         {
@@ -216,6 +241,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         // operation i of a step's OPS1: weight tile half (i < AOPS), token tile half, token scales
         auto issue_op = [&](int kb, int stage, int i) {
             const int kc = kb < nkb ? kb : nkb - 1;
+            if (TILE_PROBE(kProbeNoLoad)) return;
             if (i < AOPS) {
                 const int up = i >> 1, h = i & 1;
                 const uint8_t *src = wbase + (h * 16 + 8 * up) * p.w_rs + kc * p.w_ks + ld_chunk[h];
@@ -254,7 +280,8 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
                     lds_barrier();
                     mma_step<TH, OPS1>(a_ring + h * 8192, xbuf + h * (TM * 2048) + g * (TH * 2048),
                                        &s_xs[h][g * (TH * 16) + n], s_ws[0][kb], s_ws[1][kb], acc, frag_lo, frag_hi,
-                                       [&](int i) { issue_op(kb + 2, (h + 2) % kStages, i); });
+                                       [&](int i) { issue_op(kb + 2, (h + 2) % kStages, i); },
+                                       TILE_PROBE(kProbeNoMma));
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -407,14 +434,14 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
                     const float ws2 = s_w2s[(c0 >> 7) * n_ib + cib];
                     mma_step<THD, AOPS>(a_ring + h * 8192, aq + cib * (TMD * 2048) + g * (THD * 2048),
                                         &s_sa[cib][g * (THD * 16) + n], ws2, ws2, accd, frag_lo, frag_hi,
-                                        [&](int i) { issue2_op((h + 2) % kStages, i); });
+                                        [&](int i) { issue2_op((h + 2) % kStages, i); }, TILE_PROBE(kProbeNoMma));
                     advance2();
                     __builtin_amdgcn_sched_barrier(0);
                     cib++;
                     if (cib == n_ib) {
 #pragma unroll
                         for (int t = 0; t < THD; t++) {
-                            if (valid[t] && cg < my_groups) {
+                            if (valid[t] && cg < my_groups && !TILE_PROBE(kProbeNoY)) {
                                 uint16_t *yp = s.y + (size_t)slot[t] * K + c0 + 16 * q;
 #pragma unroll
                                 for (int half = 0; half < 2; half++) {
@@ -462,7 +489,9 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         const int left = n_live - qq * per_q;
         return left < 0 ? 0 : (left < per_q ? left : per_q);
     };
-    int qq = blockIdx.x & 7, visited = 0;
+    // (Asking for the next item's ticket while the current item runs was tried: the round trip it hides, ~2 us per item,
+    // does not show in a call's time - the kernel is bound by what all compute units pull together, not by one of them.)
+    int qq = blockIdx.x & 7, visited = 0;   // state of thread 0
     while (true) {
         if (tid == 0) {
             int it = -1;
@@ -502,10 +531,15 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         } else {
             down = (nb - lag) * per_down + (item - head_items - mid_items);
         }
-        if (up >= 0)
-            up_item(qi * per_q + up / per_up, up % per_up);
-        else
+        if (up >= 0) {
+            if (!TILE_PROBE(kProbeNoUp)) {
+                up_item(qi * per_q + up / per_up, up % per_up);
+            } else if (tid == 0) {
+                store_agent(&s.flag[(qi * per_q + up / per_up) * n_ib + up % per_up], epoch);
+            }
+        } else if (!TILE_PROBE(kProbeNoDown)) {
             run_down(qi * per_q + down / per_down, down % per_down);
+        }
         __syncthreads();   // everybody is done with the item's LDS tables and rings before the next item refills them
     }
     if (tid == 0) {
@@ -700,6 +734,7 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
     if (err != hipSuccess) return err;
     const int chunks = (p.K + 2047) / 2048;
     const int n_units = p.M * chunks;
+    if (TILE_PROBE(kProbeNoReduce)) return hipSuccess;
     hipLaunchKernelGGL(moe_tile_reduce_kernel, dim3((unsigned)(n_units < 4096 ? n_units : 4096)), dim3(256), 0, stream, s,
                        chunks, n_units);
     return hipGetLastError();
