@@ -31,7 +31,7 @@ CASES = [
     ("down items only, no result stores", NO_UP | NO_REDUCE | NO_Y),
     ("down items only, no result stores, loads without matrix work", NO_UP | NO_REDUCE | NO_Y | NO_MMA),
     ("down items only, with result stores", NO_UP | NO_REDUCE),
-    ("reduce kernel only (rows as a previous call left them)", NO_UP | NO_DOWN),
+    ("neither item kind (queue walk + reduce kernel with no live rows)", NO_UP | NO_DOWN),
 ]
 
 
