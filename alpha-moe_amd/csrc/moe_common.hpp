@@ -197,17 +197,21 @@ struct StreamCtl {
     int head;        // streaming kernel: next work item
     int done;        // streaming kernel: workgroups that have left
     int epoch;       // completed launches on this workspace (any kernel family)
-    int error;       // sticky: a bounded wait ran out
+    int pad_e;
     int fin_done;    // tile kernels: reduce-kernel workgroups that have left
     int tile_done;   // tile kernel: workgroups that have left
     int pad0[2];
     int tile_head[8];   // tile kernel: next work item of each of the eight queues
     int pad1a[16];
     // a 128-byte line of its own: idle workgroups poll it while the others still fetch items through `head`
-    int down_done;   // streaming kernel: finished DOWN items of this launch
-    int pad1[31];
+    int down_done;   // streaming kernel: finished DOWN items of this launch (+ kExpiredBit after an expired wait)
+    int error;       // sticky: a bounded wait ran out (word kErrorWord of the workspace); read with the same poll
+    int pad1[30];
 };
+constexpr int kErrorWord = 33;
 static_assert(sizeof(StreamCtl) == 256, "control block is one 256-byte line group");
+static_assert(offsetof(StreamCtl, error) == kErrorWord * sizeof(int) && offsetof(StreamCtl, down_done) % 128 == 0,
+              "the error word sits right behind the DOWN counter, on that counter's line");
 
 constexpr size_t kOffArrive = 256;
 constexpr size_t kOffFlag = kOffArrive + sizeof(int) * kMaxUnits;
@@ -218,22 +222,16 @@ constexpr size_t kPrefixBytes = kOffLive + sizeof(int) * kMaxSlots;
 // the control block instead of a hang.  The sleep grows from 0.1 us to 0.9 us: a hundred workgroups polling one address
 // every 0.2 us keep that L2 channel busy enough to slow the loads of the workgroups still streaming weights threefold
 // (measured).
-// One thread, one address:
 // "a >= b" for counters and epochs that wrap around: true while a is at most 2^31 - 1 steps ahead of b
 __device__ __forceinline__ bool reached(int a, int b) { return (int)((unsigned)a - (unsigned)b) >= 0; }
 
-__device__ __noinline__ inline void spin_until_ge(const int *addr, int target, StreamCtl *ctl)
-{
-    for (int it = 0; it < (1 << 22); it++) {
-        if (reached(load_agent(addr), target)) return;
-        if (it < 16) __builtin_amdgcn_s_sleep(4);
-        else __builtin_amdgcn_s_sleep(32);
-    }
-    store_agent(&ctl->error, 1);
-}
 // A whole wavefront, `count` <= 64 consecutive flags, one per lane: every poll is ONE load, so the wait costs one round
 // trip however many flags there are.
-__device__ __noinline__ inline void spin_all_ge(const int *addr, int count, int target, StreamCtl *ctl)
+// `also`: a counter that other workgroups are (or will be) waiting on; an expiry adds kExpiredBit to it, so that they
+// stop waiting and learn about the expiry from the very word they poll.
+constexpr int kExpiredBit = 1 << 30;
+__device__ __noinline__ inline void spin_all_ge(const int *addr, int count, int target, StreamCtl *ctl,
+                                                int *also = nullptr)
 {
     const int lane = threadIdx.x & 63;
     for (int it = 0; it < (1 << 22); it++) {
@@ -242,7 +240,10 @@ __device__ __noinline__ inline void spin_all_ge(const int *addr, int count, int 
         if (it < 16) __builtin_amdgcn_s_sleep(4);
         else __builtin_amdgcn_s_sleep(32);
     }
-    if (lane == 0) store_agent(&ctl->error, 1);
+    if (lane == 0) {
+        store_agent(&ctl->error, 1);
+        if (also) __hip_atomic_fetch_add(also, kExpiredBit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
 }
 
 // ---- tuning overrides (experiments and tests) ---------------------------------------------------------------

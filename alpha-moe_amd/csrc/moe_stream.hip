@@ -389,6 +389,9 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         activate_and_publish(u, accg, accu);
     };
 
+    // (DOWN items of two sizes - a block's last columns in quarter-size items queued behind everything else, so that
+    // the phase ends on short items - were tried: the short items stream at half the rate of the long ones, a call got
+    // 3 % slower at M = 64 and 10 % at M = 4.)
     auto down_item = [&](int item) {
         const int mb = item / s.n_cs;
         const int cs = item - mb * s.n_cs;
@@ -441,7 +444,8 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             // ring after the poll, the others before.
             if (wave != 0) prime();
 
-            if (wave == 0 && !__all(reached(flag0, epoch))) spin_all_ge(&s.flag[mb * n_ib], n_ib, epoch, s.ctl);
+            if (wave == 0 && !__all(reached(flag0, epoch)))
+                spin_all_ge(&s.flag[mb * n_ib], n_ib, epoch, s.ctl, &s.ctl->down_done);
             lds_barrier();   // the flags are up (and s_sc is written); the ring's loads stay in flight
                 if (wave == 0) prime();
 
@@ -507,47 +511,69 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         if (tid == 0) __hip_atomic_fetch_add(&s.ctl->down_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     };
 
+    // FIN item: two dependent round trips.  (1) Wavefront 0 polls the DOWN counter; an expired wait anywhere in this
+    // launch has added kExpiredBit to that very counter, and lane 1 reads the sticky error word of earlier launches
+    // with the same instruction.  (2) The stamps of the token's slots, the rows of ALL its slots and the prior output
+    // go out together; rows of slots that are not live this launch are dropped after the fact (they are stale bytes of
+    // this workspace, nothing else).
     auto fin_item = [&](int f) {
-        if (tid == 0) {
-            spin_until_ge(&s.ctl->down_done, n_down, s.ctl);
-            // A bounded wait that ran out - in this launch or in an earlier one on this workspace: the word is sticky -
-            // means that some result rows may be missing.  The output then says so itself: NaN in every element.
-            // One thread asks (agent-scope loads of one word from every wavefront queue up at the memory side).
-            s_bcast[1] = load_agent(&s.ctl->error);
+        if (wave == 0) {
+            int v = 0;
+            bool up = false;
+            for (int it = 0; it < (1 << 22) && !up; it++) {
+                v = load_agent(lane == 1 ? &s.ctl->error : &s.ctl->down_done);
+                up = reached(__builtin_amdgcn_readlane(v, 0), n_down);
+                if (!up) {
+                    if (it < 16) __builtin_amdgcn_s_sleep(4);
+                    else __builtin_amdgcn_s_sleep(32);
+                }
+            }
+            if (lane == 0) {
+                if (!up) store_agent(&s.ctl->error, 1);
+                // a result row may be missing: the output says so itself, NaN in every element
+                s_bcast[1] = !up || __builtin_amdgcn_readlane(v, 1) != 0 || (__builtin_amdgcn_readlane(v, 0) >> 30) != 0;
+            }
         }
         __syncthreads();
         const int t = f / s.n_fc;
         const int c = (f - t * s.n_fc) * kFinCols + tid * 4;
-        // lane k fetches the stamp of the token's slot k: one round trip for all of them (top_k <= 64)
-        const int stamp = load_agent(&s.live[t * p.top_k + (lane < p.top_k ? lane : 0)]);
+        const bool mine = tid < kFinCols / 4 && c < K;
         const bool poisoned = s_bcast[1] != 0;
-        const unsigned long long live_mask = __ballot(lane < p.top_k && stamp == epoch);
-        if (poisoned) {
-            if (tid < kFinCols / 4 && c < K)
-                *reinterpret_cast<uint2 *>(p.out + (size_t)t * K + c) = make_uint2(0x7fc07fc0u, 0x7fc07fc0u);
-        } else if (tid < kFinCols / 4 && c < K) {
-            v4f sum = {0.f, 0.f, 0.f, 0.f};
-            // slot order: the sum depends on nothing but the inputs.  Eight rows are in flight at a time.
-            for (int s0 = 0; s0 < p.top_k; s0 += 8) {
-                v4i bits[8];
+        // lane k fetches the stamp of the token's slot k (top_k <= 64)
+        const int stamp = load_agent(&s.live[t * p.top_k + (lane < p.top_k ? lane : 0)]);
+        uint2 *op = reinterpret_cast<uint2 *>(p.out + (size_t)t * K + (mine ? c : 0));
+        uint2 o = {0u, 0u};
+        if (mine && !p.overwrite && !poisoned) o = *op;
+        v4f sum = {0.f, 0.f, 0.f, 0.f};
+        // slot order: the sum depends on nothing but the inputs.  Sixteen rows are in flight at a time.
+        for (int s0 = 0; s0 < p.top_k; s0 += 16) {
+            v4i lo[8], hi[8];
 #pragma unroll
-                for (int k = 0; k < 8; k++) {
-                    const int slot = t * p.top_k + s0 + k;
-                    const bool on = s0 + k < p.top_k && ((live_mask >> (s0 + k)) & 1);
-                    bits[k] = (v4i){0, 0, 0, 0};
-                    if (on) bits[k] = ldg128_agent(s.y + (size_t)slot * K + c);
-                }
-                drain_vmem_into(bits);
-#pragma unroll
-                for (int k = 0; k < 8; k++) sum += __builtin_bit_cast(v4f, bits[k]);
+            for (int k = 0; k < 8; k++) {
+                lo[k] = (v4i){0, 0, 0, 0};
+                hi[k] = (v4i){0, 0, 0, 0};
+                if (mine && s0 + k < p.top_k) lo[k] = ldg128_agent(s.y + (size_t)(t * p.top_k + s0 + k) * K + c);
+                if (mine && s0 + 8 + k < p.top_k) hi[k] = ldg128_agent(s.y + (size_t)(t * p.top_k + s0 + 8 + k) * K + c);
             }
-            uint2 *op = reinterpret_cast<uint2 *>(p.out + (size_t)t * K + c);
-            uint2 o = {0u, 0u};
-            if (!p.overwrite) o = *op;
-            const float o0 = __builtin_bit_cast(float, o.x << 16), o1 = __builtin_bit_cast(float, o.x & 0xffff0000u);
-            const float o2 = __builtin_bit_cast(float, o.y << 16), o3 = __builtin_bit_cast(float, o.y & 0xffff0000u);
-            o.x = pack_bf16x2(o0 + sum[0], o1 + sum[1]);
-            o.y = pack_bf16x2(o2 + sum[2], o3 + sum[3]);
+            drain_vmem_into(lo);
+            drain_vmem_into(hi);
+            const unsigned long long live_mask = __ballot(lane < p.top_k && stamp == epoch) >> s0;
+#pragma unroll
+            for (int k = 0; k < 8; k++)
+                if ((live_mask >> k) & 1) sum += __builtin_bit_cast(v4f, lo[k]);
+#pragma unroll
+            for (int k = 0; k < 8; k++)
+                if ((live_mask >> (8 + k)) & 1) sum += __builtin_bit_cast(v4f, hi[k]);
+        }
+        if (mine) {
+            if (poisoned) {
+                o = make_uint2(0x7fc07fc0u, 0x7fc07fc0u);
+            } else {
+                const float o0 = __builtin_bit_cast(float, o.x << 16), o1 = __builtin_bit_cast(float, o.x & 0xffff0000u);
+                const float o2 = __builtin_bit_cast(float, o.y << 16), o3 = __builtin_bit_cast(float, o.y & 0xffff0000u);
+                o.x = pack_bf16x2(o0 + sum[0], o1 + sum[1]);
+                o.y = pack_bf16x2(o2 + sum[2], o3 + sum[3]);
+            }
             *op = o;
         }
     };

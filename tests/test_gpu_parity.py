@@ -462,7 +462,8 @@ def test_workspace_check_reports_an_expired_wait(c1):
     for knobs in ((16, 32, 8, 5), (64, 64, 4, 3)):
         assert_parity(run_op(P, *knobs, via="c_abi", workspace=ws), ref, f"knobs {knobs}")
         assert alpha_moe.c_abi.alpha_moe_workspace_check(ws.data_ptr(), stream) == 0
-    ws.view(torch.int32)[3] = 1   # the control block's error word
+    error_word = 33   # the control block's sticky error word (kErrorWord in csrc/moe_common.hpp)
+    ws.view(torch.int32)[error_word] = 1
     rc = alpha_moe.c_abi.alpha_moe_workspace_check(ws.data_ptr(), stream)
     assert rc == 8 and b"wait" in alpha_moe.c_abi.alpha_moe_status_string(rc)
     # while the word is set, every call on the workspace says so in its output: NaN everywhere, adding or storing,
@@ -471,7 +472,7 @@ def test_workspace_check_reports_an_expired_wait(c1):
         for store in (False, True):
             got = run_op(P, *knobs, via="c_abi", workspace=ws, store=store)
             assert torch.isnan(got.float()).all(), (knobs, store)
-    ws.view(torch.int32)[3] = 0
+    ws.view(torch.int32)[error_word] = 0
     assert_parity(run_op(P, 16, 32, 8, 5, via="c_abi", workspace=ws), ref, "after clearing the error word")
 
 
