@@ -396,8 +396,9 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         const int mb = item / s.n_cs;
         const int cs = item - mb * s.n_cs;
         const Routing<TM> r = load_routing<TM>(p, mb, n);   // in flight together with the expert id
-        // so is a first look at the flags of the block's slices (one lane each)
-        const int flag0 = (wave == 0 && lane < s.n_ib) ? load_agent(&s.flag[mb * s.n_ib + lane]) : epoch;
+        // so is every wavefront's own look at the flags of the block's slices (one lane each): a wavefront that has seen
+        // them up may read what the UP items published without meeting the others first
+        const int flag0 = lane < s.n_ib ? load_agent(&s.flag[mb * s.n_ib + lane]) : epoch;
         const int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
         if (e >= 0 && e < p.E) {
             const int n_ib = s.n_ib;
@@ -434,20 +435,21 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                     slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
                 }
             };
-            // w2 scales of the 128-column blocks this item touches: s_sc[blk * n_ib + ib].  Loaded BEFORE the ring is
-            // filled: waiting for them then leaves the ring's loads in flight.
+            // Everything the item needs goes out before anything is waited for: the w2 scales of the 128-column blocks
+            // the item touches (s_sc[blk * n_ib + ib], at most four per thread), the ring's first tiles, and - once
+            // this wavefront has seen the flags up - the requantised activations and their scales.
             const int blk0 = (t0 * 16) >> 7;
             const int nblk = (((t1 * 16) - 1) >> 7) - blk0 + 1;
-            for (int i = tid; i < nblk * n_ib; i += THREADS)
-                s_sc[i] = p.w2_scale[((size_t)e * (K >> 7) + blk0) * n_ib + i];
-            // Wavefront 0 polls the flags, and a poll returns behind everything the wavefront has in flight: it fills its
-            // ring after the poll, the others before.
-            if (wave != 0) prime();
-
-            if (wave == 0 && !__all(reached(flag0, epoch)))
-                spin_all_ge(&s.flag[mb * n_ib], n_ib, epoch, s.ctl, &s.ctl->down_done);
-            lds_barrier();   // the flags are up (and s_sc is written); the ring's loads stay in flight
-                if (wave == 0) prime();
+            const float *w2s = p.w2_scale + ((size_t)e * (K >> 7) + blk0) * n_ib;
+            float sc_reg[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int i = tid + k * THREADS;
+                sc_reg[k] = i < nblk * n_ib ? w2s[i] : 0.f;
+            }
+            prime();
+            // rare (a DOWN item is queued long after the UP items it needs): a poll returns behind the ring's loads
+            if (!__all(reached(flag0, epoch))) spin_all_ge(&s.flag[mb * n_ib], n_ib, epoch, s.ctl, &s.ctl->down_done);
 
             // requantised activations of all slices -> LDS as operand tiles, their scales -> s_xs[row][ib]
             for (int i = wave; i < n_ib * TM; i += WN) {
@@ -457,10 +459,14 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 for (int k = 0; k < 2; k++)
                     dma16<16>(src + (8 * k + ld_row) * 128 + 16 * ld_chunk[k], s_aq + i * 2048 + k * 1024);
             }
-            for (int i = tid; i < n_ib * TM * 16; i += THREADS) {
+            static_assert(kMaxIb * TM * 16 <= 2 * THREADS, "at most two activation scales per thread");
+            int sa_bits[2] = {0, 0};
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const int i = tid + k * THREADS;
                 const int ib = i / (TM * 16), row = i - ib * (TM * 16);
-                const int bits = load_agent(reinterpret_cast<const int *>(&s.sa[(size_t)(mb * n_ib + ib) * s.bm_pad + row]));
-                s_xs[row][ib] = __builtin_bit_cast(float, bits);
+                if (i < n_ib * TM * 16)
+                    sa_bits[k] = load_agent(reinterpret_cast<const int *>(&s.sa[(size_t)(mb * n_ib + ib) * s.bm_pad + row]));
             }
             float tw[TM];
             float *yp[TM];
@@ -469,6 +475,17 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 tw[t] = r.valid[t] ? p.topk_w[r.slot[t]] * p.scaling : 0.f;
                 yp[t] = s.y + (size_t)r.slot[t] * K + 4 * q;
                 if (cs == 0 && wave == 0 && q == 0 && r.valid[t]) store_agent(&s.live[r.slot[t]], epoch);
+            }
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int i = tid + k * THREADS;
+                if (i < nblk * n_ib) s_sc[i] = sc_reg[k];
+            }
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const int i = tid + k * THREADS;
+                const int ib = i / (TM * 16), row = i - ib * (TM * 16);
+                if (i < n_ib * TM * 16) s_xs[row][ib] = __builtin_bit_cast(float, sa_bits[k]);
             }
             // everything issued so far (the ring's first S-1 tiles, the activation tiles) has landed
             drain_vmem();
