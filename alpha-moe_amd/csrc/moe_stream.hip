@@ -491,37 +491,50 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             drain_vmem();
             __syncthreads();
 
-            v4f d[TM];
+            // Result rows are kept in registers and stored NG column groups at a time, normally once, behind the
+            // item's last tile: the wait counter that tells a wavefront that a ring tile has landed counts stores as
+            // well, in issue order, so a store between the loads holds every later tile back until it is acknowledged
+            // by memory (measured on the DeepSeek-V3 shard at M = 64: 234 -> 215 us per call with the stores taken out).
+            constexpr int NG = 16 / TM;
+            for (int g0 = 0; g0 < wng; g0 += NG) {
+                v4f res[NG][TM];
 #pragma unroll
-            for (int t = 0; t < TM; t++) d[t] = (v4f){0.f, 0.f, 0.f, 0.f};
-            int cg = 0, cib = 0;   // (group, slice) of the tile being consumed
-            for (int j = 0; j < wnt; j++) {
-                issue(slot_w);
-                slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
-                __builtin_amdgcn_sched_barrier(0);
-                wait_vmcnt<2 * (S - 1)>();
-                const v8i a = read_tile(ring + slot_r * 2048);
-                slot_r = slot_r + 1 == S ? 0 : slot_r + 1;
-                const int c0 = (wt0 + cg) << 4;
-                const float ws = s_sc[((c0 >> 7) - blk0) * n_ib + cib];
+                for (int gg = 0; gg < NG; gg++) {
+                    if (g0 + gg < wng) {   // wavefront-uniform
+                        const int c0 = (wt0 + g0 + gg) << 4;
+                        v4f d[TM];
 #pragma unroll
-                for (int t = 0; t < TM; t++) {
-                    const v8i b = read_tile(s_aq + (cib * TM + t) * 2048);
-                    d[t] += mfma_fp8(a, b) * (s_xs[t * 16 + n][cib] * ws);
-                }
-                cib++;
-                if (cib == n_ib) {
-                    cib = 0;
-                    cg++;
+                        for (int t = 0; t < TM; t++) d[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+                        for (int cib = 0; cib < n_ib; cib++) {
+                            issue(slot_w);
+                            slot_w = slot_w + 1 == S ? 0 : slot_w + 1;
+                            __builtin_amdgcn_sched_barrier(0);
+                            wait_vmcnt<2 * (S - 1)>();
+                            const v8i a = read_tile(ring + slot_r * 2048);
+                            slot_r = slot_r + 1 == S ? 0 : slot_r + 1;
+                            const float ws = s_sc[((c0 >> 7) - blk0) * n_ib + cib];
 #pragma unroll
-                    for (int t = 0; t < TM; t++) {
-                        if (r.valid[t]) stg128_agent(yp[t] + c0, d[t] * tw[t]);
-                        d[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+                            for (int t = 0; t < TM; t++) {
+                                const v8i b = read_tile(s_aq + (cib * TM + t) * 2048);
+                                d[t] += mfma_fp8(a, b) * (s_xs[t * 16 + n][cib] * ws);
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+#pragma unroll
+                        for (int t = 0; t < TM; t++) res[gg][t] = d[t] * tw[t];
                     }
                 }
-                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int gg = 0; gg < NG; gg++)
+                    if (g0 + gg < wng) {
+#pragma unroll
+                        for (int t = 0; t < TM; t++)
+                            if (r.valid[t]) stg128_agent(yp[t] + ((wt0 + g0 + gg) << 4), res[gg][t]);
+                    }
             }
         }
+        // (Asking for the next item when the last tile is issued, and counting the item only behind the next item's
+        // prologue instead of waiting for its rows here, were both tried: 1 - 3 % slower at M = 16 and 64.)
         fetch_next();
         drain_vmem();
         __syncthreads();
