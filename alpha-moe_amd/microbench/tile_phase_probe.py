@@ -82,10 +82,12 @@ def main():
     ap.add_argument("--M", type=int, default=8192)
     ap.add_argument("--block-m", type=int, default=128)
     ap.add_argument("--calls", type=int, default=8)
+    ap.add_argument("--bits", type=int, nargs="*", help="only the cases with these bits (e.g. under rocprofv3 --pmc)")
     args = ap.parse_args()
     tmp = tempfile.mkdtemp(prefix="alpha_moe_probe_")
+    cases = [c for c in CASES if args.bits is None or c[1] in args.bits]
     print("building one library per case ...", flush=True)
-    libs = {mask: bind(path) for mask, path in build_probe_libraries(tmp, [m for _, m in CASES]).items()}
+    libs = {mask: bind(path) for mask, path in build_probe_libraries(tmp, sorted({0} | {m for _, m in cases})).items()}
     lib = libs[0]
     dev = "cuda:0"
     W = make_weights(SHAPES[args.shape], device=dev, seed=0)
@@ -108,7 +110,7 @@ def main():
 
     print(f"{args.shape} M={args.M} block_m={args.block_m}: median of {args.calls} calls, each behind a 512 MiB fill")
     print(f"algorithmic flops {P.algorithmic_flops() / 1e9:.1f} G, bytes {P.algorithmic_bytes() / 1e6:.1f} MB")
-    for name, mask in CASES:
+    for name, mask in cases:
         call(libs[mask])
         torch.cuda.synchronize()
         ts = []
