@@ -33,7 +33,7 @@ sys.path.insert(0, ROOT)
 # configurations that were profiled (all kernels of a call):
 #   profiles/moe_stream_kernel_ds_decode_M64_hbm_traffic.md, profiles/moe_tile_kernel_ds_prefill_M8192_hbm_traffic.md,
 #   profiles/moe_tile_kernel_q3_prefill_M8192_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES = {("ds", 64): 1293.9e6, ("ds", 512): 1676.0e6, ("ds", 2048): 2240.8e6, ("ds", 8192): 4802.9e6,
+MEASURED_TRAFFIC_BYTES = {("ds", 64): 1293.5e6, ("ds", 512): 1676.0e6, ("ds", 2048): 2240.8e6, ("ds", 8192): 4802.9e6,
                           ("q3", 1024): 813.4e6, ("q3", 8192): 1897.0e6}
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
