@@ -66,7 +66,8 @@ struct StreamPlan {
     int n_ib, nkb, n_ct, n_mb_max;
     int kbpi, ks;    // K blocks per UP item, UP items per unit
     int tpi, n_cs;   // 16-column tiles per DOWN item, DOWN items per row block
-    int n_fc;        // FIN items per token
+    int n_fc;        // 1024-column chunks per token
+    int fin_w;       // chunks per FIN item (1 or 2)
     int lag;         // row blocks between a block's UP items and its DOWN items in the queue
     int bm_pad;
     int strict_queue;   // every item, the first one too, comes from the counter: correct with any number of resident workgroups
@@ -175,7 +176,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     const int n_units = n_mb * s.n_ib;
     const int n_up = n_units * s.ks;
     const int n_down = n_mb * s.n_cs;
-    const int n_fin = p.M * s.n_fc;
+    const int n_fin = (p.M * s.n_fc + s.fin_w - 1) / s.fin_w;
     const int total = n_up + n_down + n_fin;
     const int epoch = (int)((unsigned)__builtin_amdgcn_readfirstlane(s.ctl->epoch) + 1u);
     const uint8_t *dummy = p.x;   // where loads past the end of an item are pointed: always mapped, always cached
@@ -595,47 +596,71 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         }
         __syncthreads();
         TRACE_MARK;
-        const int t = f / s.n_fc;
-        const int c = (f - t * s.n_fc) * kFinCols + tid * 4;
-        const bool mine = tid < kFinCols / 4 && c < K;
+        // an item sums fin_w (1 or 2) chunks of 1024 columns: with more chunks than workgroups, two per item halve the
+        // rounds of dependent memory round trips that close the call
         const bool poisoned = s_bcast[1] != 0;
-        // lane k fetches the stamp of the token's slot k (top_k <= 64)
-        const int stamp = load_agent(&s.live[t * p.top_k + (lane < p.top_k ? lane : 0)]);
-        uint2 *op = reinterpret_cast<uint2 *>(p.out + (size_t)t * K + (mine ? c : 0));
-        uint2 o = {0u, 0u};
-        if (mine && !p.overwrite && !poisoned) o = *op;
-        v4f sum = {0.f, 0.f, 0.f, 0.f};
-        // slot order: the sum depends on nothing but the inputs.  Sixteen rows are in flight at a time.
+        const int n_chunks = p.M * s.n_fc;
+        int tk[2], col[2], stamp[2];
+        bool mine[2];
+        uint2 *op[2];
+        uint2 o[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int ch = f * s.fin_w + j;
+            const bool on = j < s.fin_w && ch < n_chunks;
+            tk[j] = on ? ch / s.n_fc : 0;
+            col[j] = (on ? ch - tk[j] * s.n_fc : 0) * kFinCols + tid * 4;
+            mine[j] = on && tid < kFinCols / 4 && col[j] < K;
+            // lane k fetches the stamp of the token's slot k (top_k <= 64)
+            stamp[j] = load_agent(&s.live[tk[j] * p.top_k + (lane < p.top_k ? lane : 0)]);
+            op[j] = reinterpret_cast<uint2 *>(p.out + (size_t)tk[j] * K + (mine[j] ? col[j] : 0));
+            o[j] = make_uint2(0u, 0u);
+            if (mine[j] && !p.overwrite && !poisoned) o[j] = *op[j];
+        }
+        v4f sum[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        // slot order: the sum depends on nothing but the inputs.  Sixteen rows per chunk are in flight at a time.
         for (int s0 = 0; s0 < p.top_k; s0 += 16) {
-            v4i lo[8], hi[8];
+            v4i lo[2][8], hi[2][8];
 #pragma unroll
-            for (int k = 0; k < 8; k++) {
-                lo[k] = (v4i){0, 0, 0, 0};
-                hi[k] = (v4i){0, 0, 0, 0};
-                if (mine && s0 + k < p.top_k) lo[k] = ldg128_agent(s.y + (size_t)(t * p.top_k + s0 + k) * K + c);
-                if (mine && s0 + 8 + k < p.top_k) hi[k] = ldg128_agent(s.y + (size_t)(t * p.top_k + s0 + 8 + k) * K + c);
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    lo[j][k] = (v4i){0, 0, 0, 0};
+                    hi[j][k] = (v4i){0, 0, 0, 0};
+                    const float *row = s.y + (size_t)(tk[j] * p.top_k + s0 + k) * K + col[j];
+                    if (mine[j] && s0 + k < p.top_k) lo[j][k] = ldg128_agent(row);
+                    if (mine[j] && s0 + 8 + k < p.top_k) hi[j][k] = ldg128_agent(row + (size_t)8 * K);
+                }
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                drain_vmem_into(lo[j]);
+                drain_vmem_into(hi[j]);
             }
-            drain_vmem_into(lo);
-            drain_vmem_into(hi);
-            const unsigned long long live_mask = __ballot(lane < p.top_k && stamp == epoch) >> s0;
 #pragma unroll
-            for (int k = 0; k < 8; k++)
-                if ((live_mask >> k) & 1) sum += __builtin_bit_cast(v4f, lo[k]);
+            for (int j = 0; j < 2; j++) {
+                const unsigned long long live_mask = __ballot(lane < p.top_k && stamp[j] == epoch) >> s0;
 #pragma unroll
-            for (int k = 0; k < 8; k++)
-                if ((live_mask >> (8 + k)) & 1) sum += __builtin_bit_cast(v4f, hi[k]);
-        }
-        if (mine) {
-            if (poisoned) {
-                o = make_uint2(0x7fc07fc0u, 0x7fc07fc0u);
-            } else {
-                const float o0 = __builtin_bit_cast(float, o.x << 16), o1 = __builtin_bit_cast(float, o.x & 0xffff0000u);
-                const float o2 = __builtin_bit_cast(float, o.y << 16), o3 = __builtin_bit_cast(float, o.y & 0xffff0000u);
-                o.x = pack_bf16x2(o0 + sum[0], o1 + sum[1]);
-                o.y = pack_bf16x2(o2 + sum[2], o3 + sum[3]);
+                for (int k = 0; k < 8; k++)
+                    if ((live_mask >> k) & 1) sum[j] += __builtin_bit_cast(v4f, lo[j][k]);
+#pragma unroll
+                for (int k = 0; k < 8; k++)
+                    if ((live_mask >> (8 + k)) & 1) sum[j] += __builtin_bit_cast(v4f, hi[j][k]);
             }
-            *op = o;
         }
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+            if (mine[j]) {
+                uint2 r = o[j];
+                if (poisoned) {
+                    r = make_uint2(0x7fc07fc0u, 0x7fc07fc0u);
+                } else {
+                    const float o0 = __builtin_bit_cast(float, r.x << 16), o1 = __builtin_bit_cast(float, r.x & 0xffff0000u);
+                    const float o2 = __builtin_bit_cast(float, r.y << 16), o3 = __builtin_bit_cast(float, r.y & 0xffff0000u);
+                    r.x = pack_bf16x2(o0 + sum[j][0], o1 + sum[j][1]);
+                    r.y = pack_bf16x2(o2 + sum[j][2], o3 + sum[j][3]);
+                }
+                *op[j] = r;
+            }
     };
 
     // ---- work queue ---------------------------------------------------------------------------------------
@@ -707,7 +732,7 @@ size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
 struct HostPlan {
     bool ok;
     int bm_pad, n_ib, nkb, n_ct, n_mb_max, units;
-    int kbpi, ks, tpi, n_cs, n_fc, lag;
+    int kbpi, ks, tpi, n_cs, n_fc, fin_w, lag;
     size_t off_sa, off_aq, off_hpart, off_y, total;
 };
 
@@ -776,6 +801,7 @@ HostPlan make_plan(int top_k, int M, int K, int N, int E, int sorted_num, int bl
     h.tpi = ((h.n_ct + h.n_cs - 1) / h.n_cs + 15) / 16 * 16;   // even split, whole multiples of 16 tiles
     h.n_cs = (h.n_ct + h.tpi - 1) / h.tpi;
     h.n_fc = (K + kFinCols - 1) / kFinCols;
+    h.fin_w = (int64_t)M * h.n_fc > cus ? 2 : 1;
     // how many row blocks later a block's DOWN items enter the queue than its UP items
     // (measured: overlapping the two kinds lowers the total rate - DOWN items stream less efficiently than UP items -
     // so by default the lag is "all blocks", i.e. UP items first, then DOWN items)
@@ -933,6 +959,7 @@ hipError_t launch_stream(const MoeParams &p, int warp_n, int stages, void *works
     s.tpi = h.tpi;
     s.n_cs = h.n_cs;
     s.n_fc = h.n_fc;
+    s.fin_w = h.fin_w;
     s.lag = h.lag;
     s.strict_queue = tunable(kTunStrictQueue, 1) != 0;
 
