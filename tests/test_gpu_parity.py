@@ -474,6 +474,15 @@ def test_workspace_check_reports_an_expired_wait(c1):
             assert torch.isnan(got.float()).all(), (knobs, store)
     ws.view(torch.int32)[error_word] = 0
     assert_parity(run_op(P, 16, 32, 8, 5, via="c_abi", workspace=ws), ref, "after clearing the error word")
+    # An expiry DURING a launch of the streaming kernel reaches the closing items through the counter they poll: the
+    # waiter adds a high bit to it.  Set from the host here, the bit makes that one launch answer NaN (its closing items
+    # do not wait and do not trust what they read); the launch resets the counter, and the next one is clean again.
+    down_counter, expired_bit = 32, 1 << 30   # StreamCtl::down_done and kExpiredBit in csrc/moe_common.hpp
+    ws.view(torch.int32)[down_counter] = expired_bit
+    got = run_op(P, 16, 32, 8, 5, via="c_abi", workspace=ws)
+    assert torch.isnan(got.float()).all()
+    assert_parity(run_op(P, 16, 32, 8, 5, via="c_abi", workspace=ws), ref, "the launch after a marked counter")
+    assert alpha_moe.c_abi.alpha_moe_workspace_check(ws.data_ptr(), stream) == 0
 
 
 def test_queue_survives_a_grid_the_device_cannot_hold(ds_weights):
