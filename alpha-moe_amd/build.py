@@ -33,6 +33,7 @@ HIP_SOURCES = {
     "moe_direct.hip": [],
     "moe_stream.hip": [],
     "moe_tile.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+    "moe_wide.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
     "moe_prep.hip": [],
 }
 

@@ -30,7 +30,7 @@ void load_tunables_once()
             const char *e = getenv(t.name);
             if (!e) continue;
             if (!strcmp(t.name, "ALPHA_MOE_PATH"))
-                t.value = !strcmp(e, "direct") ? 1 : !strcmp(e, "stream") ? 2 : !strcmp(e, "tile") ? 3 : kTunableUnset;
+                t.value = !strcmp(e, "direct") ? 1 : !strcmp(e, "stream") ? 2 : !strcmp(e, "tile") ? 3 : !strcmp(e, "wide") ? 4 : kTunableUnset;
             else
                 t.value = atoi(e);
         }
@@ -39,19 +39,23 @@ void load_tunables_once()
     (void)done;
 }
 
-enum Path { kDirect, kStream, kTile };
+enum Path { kDirect, kStream, kTile, kWide };
 
-// Streaming kernel for row blocks of at most 32 rows (decode), tile kernel above (prefill); the direct kernel is the
-// fallback for shapes neither takes.
-Path choose_path(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
+// Streaming kernel for row blocks of at most 32 rows (decode); above that (prefill) warp_n picks the token tiles a
+// wavefront multiplies per step: 8 -> wide kernel (macro blocks of 256 rows), 4 -> tile kernel (one row block).  The
+// direct kernel is the fallback for shapes none of them takes.
+Path choose_path(int top_k, int M, int K, int N, int E, int sorted_num, int block_m, int warp_n)
 {
     const bool s_ok = stream_supported(top_k, M, K, N, E, sorted_num, block_m);
     const bool t_ok = tile_supported(top_k, M, K, N, E, sorted_num, block_m);
+    const bool w_ok = wide_supported(top_k, M, K, N, E, sorted_num, block_m);
     const int f = tunable(kTunPath, 0);
     if (f == 1) return kDirect;
     if (f == 2 && s_ok) return kStream;
     if (f == 3 && t_ok) return kTile;
+    if (f == 4 && w_ok) return kWide;
     if (s_ok) return kStream;
+    if (w_ok && (warp_n == 8 || !t_ok)) return kWide;
     if (t_ok) return kTile;
     return kDirect;
 }
@@ -104,8 +108,12 @@ extern "C" size_t alpha_moe_workspace_bytes(int top_k, int M, int K, int N, int 
     const size_t tile = tile_supported(top_k, M, K, N, num_experts, sorted_num, block_m)
                             ? tile_workspace_bytes(top_k, M, K, N, num_experts, sorted_num, block_m)
                             : 0;
-    const size_t m = direct > stream ? direct : stream;
-    return m > tile ? m : tile;
+    const size_t wide = wide_supported(top_k, M, K, N, num_experts, sorted_num, block_m)
+                            ? wide_workspace_bytes(top_k, M, K, N, num_experts, sorted_num, block_m)
+                            : 0;
+    size_t m = direct > stream ? direct : stream;
+    m = m > tile ? m : tile;
+    return m > wide ? m : wide;
 }
 
 namespace {
@@ -143,9 +151,11 @@ int run_fused_moe(const uint8_t *x, const float *x_scale, const uint8_t *w, cons
 
     hipStream_t hs = static_cast<hipStream_t>(stream);
     hipError_t err;
-    const Path path = choose_path(top_k, M, K, N, num_experts, sorted_num, block_m);
+    const Path path = choose_path(top_k, M, K, N, num_experts, sorted_num, block_m, warp_n);
     if (path == kStream) {
         err = launch_stream(p, warp_n, stages, workspace, hs);
+    } else if (path == kWide) {
+        err = launch_wide(p, workspace, hs);
     } else if (path == kTile) {
         err = launch_tile(p, workspace, hs);
     } else {

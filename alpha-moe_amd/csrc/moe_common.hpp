@@ -289,4 +289,20 @@ bool tile_supported(int top_k, int M, int K, int N, int E, int sorted_num, int b
 size_t tile_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
 hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream);
 
+// Wide kernel for large batches: macro blocks of up to 256 consecutive sorted rows of one expert (several row blocks),
+// twice the tokens per weight byte of the tile kernel; same per-slot result rows and reduce kernel.  block_m > 32.
+bool wide_supported(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
+size_t wide_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
+hipError_t launch_wide(const MoeParams &p, void *workspace, hipStream_t stream);
+
+// out[t] = bf16(out[t] + sum over the token's live slots of y[slot]) (or bf16(sum) when p.overwrite); closes the
+// workspace's launch epoch.  Shared by the tile and wide kernels, which write each (token, slot) row once into y.
+struct RowsReduce {
+    MoeParams p;
+    StreamCtl *ctl;
+    const int *live;      // [slots] == epoch + 1 of the control block for rows written in this launch
+    const uint16_t *y;    // [slots][K] bf16
+};
+hipError_t launch_rows_reduce(const RowsReduce &r, hipStream_t stream);
+
 }  // namespace alpha_moe

@@ -554,7 +554,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
 // out[t] = bf16(out[t] + sum over the token's live slots of y[slot]); the last workgroup to leave closes the epoch.
 // A unit is (token, 2048 columns): a thread owns 8 columns and keeps up to 8 row loads in flight.  Workgroups stride
 // over the units so that the closing counter sees a few thousand arrivals, not one per unit.
-__global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams s, int chunks_per_token, int n_units)
+__global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const RowsReduce s, int chunks_per_token, int n_units)
 {
     const MoeParams &p = s.p;
     const int epoch = (int)((unsigned)s.ctl->epoch + 1u);
@@ -732,10 +732,20 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
     hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(512), lds_bytes, stream, s);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
-    const int chunks = (p.K + 2047) / 2048;
-    const int n_units = p.M * chunks;
     if (TILE_PROBE(kProbeNoReduce)) return hipSuccess;
-    hipLaunchKernelGGL(moe_tile_reduce_kernel, dim3((unsigned)(n_units < 4096 ? n_units : 4096)), dim3(256), 0, stream, s,
+    RowsReduce r;
+    r.p = p;
+    r.ctl = s.ctl;
+    r.live = s.live;
+    r.y = s.y;
+    return launch_rows_reduce(r, stream);
+}
+
+hipError_t launch_rows_reduce(const RowsReduce &r, hipStream_t stream)
+{
+    const int chunks = (r.p.K + 2047) / 2048;
+    const int n_units = r.p.M * chunks;
+    hipLaunchKernelGGL(moe_tile_reduce_kernel, dim3((unsigned)(n_units < 4096 ? n_units : 4096)), dim3(256), 0, stream, r,
                        chunks, n_units);
     return hipGetLastError();
 }

@@ -1,0 +1,779 @@
+// Fused W8A8 MoE, "wide" kernel for large batches: the work unit is a MACRO BLOCK of up to 256 consecutive sorted rows
+// of one expert (as many whole row blocks of block_m rows as fit), not a single row block.
+//
+// Why: on MI355X the tile kernel's up/gate items spend their time bringing operands to LDS, not multiplying them.  A
+// 256-row weight slab against 128 tokens is 48 KiB through L2 per 128-byte K step for 8.4 MFLOP; against 256 tokens it
+// is 64 KiB for 16.8 MFLOP, a third fewer bytes per flop, and the weight bytes - the ones that miss L2 because an
+// expert's slab is streamed once - are halved.  The 256 x 256 fp32 accumulators are 128 registers of each of the
+// workgroup's eight wavefronts, which is what the register file holds next to the operands.
+//
+// Persistent workgroups of 8 wavefronts (two per SIMD, one workgroup per compute unit) take items from eight queues,
+// one per XCD, exactly as in the tile kernel.  A macro block is I/128 UP items (one 128-column slice each) and a few
+// DOWN items (a slab of output columns each).  Which row blocks form a macro block is decided on the device by
+// moe_wide_plan_kernel (the host does not know expert_ids): consecutive blocks of one expert, floor(256 / block_m) at
+// a time.
+//
+// Wavefront (w, g): weight rows 64 w .. 64 w + 63 (four operand tiles, shared with the pair's other wavefront through
+// a two-stage LDS ring), token tiles g, g + 2, ..., g + 14 (interleaved so that a partly filled macro block loads
+// both wavefronts of a pair alike).  Token tiles past the block's last valid row are neither loaded nor multiplied.
+// Two ring stages of 64 KiB (32 KiB of weights, 32 KiB of tokens): the loads of step k + 1 are issued while step k
+// is multiplied, and one workgroup barrier per step orders everything.
+//
+// UP item: SwiGLU and the FP8 requantisation of the 128-column group in registers, operand tiles + per-token scales
+// to scratch, then the unit's flag (fused_moe_w8a8_up_down_acc.cu:863-994 of the reference).  DOWN item: waits for
+// the flags of the block's slices and contracts their tiles with w2, 64 output columns per pair of wavefronts and
+// step; the tiles either sit in LDS for the whole item (I/128 <= 2: they fit where the token ring was) or stream
+// through the ring like tokens do.  Each valid (token, slot) row is written once, bf16, whole 128-byte lines, to
+// y[slot]; the tile kernel's reduce kernel sums a token's rows in fp32 and rounds into `out` once
+// (fused_moe_w8a8_up_down_acc.cu:1007-1096 adds top_k * I/128 partial rows per token into the output instead).
+#include <mutex>
+#include <type_traits>
+
+#include "moe_common.hpp"
+
+namespace alpha_moe {
+namespace {
+
+constexpr int kWRows = 256;                 // token rows of a macro block
+constexpr int kWTiles = kWRows / 16;        // 16-token operand tiles of a macro block
+constexpr int kWStageA = 4 * 4 * 2048;      // 4 pairs x 4 weight tiles of 2 KiB
+constexpr int kWStageX = kWTiles * 2048;    // 16 token tiles
+constexpr int kWDynLds = 2 * kWStageA + 2 * kWStageX;
+constexpr int kWMaxKb = 128;                // most 128-byte K blocks (K <= 16384)
+constexpr int kWMaxW2s = 1024;              // most w2 block scales of one expert, (K/128) * (I/128)
+constexpr int kWResidentIb = 2;             // slices whose requantised tiles fit LDS for a whole DOWN item
+
+struct WideParams {
+    MoeParams p;
+    StreamCtl *ctl;
+    int *flag;        // [first row block of a macro block][n_ib] == epoch once the slice's tiles are in scratch
+    int *live;        // [slots] == epoch once y[slot] is written this launch
+    uint16_t *y;      // [slots][K] bf16
+    uint8_t *aqs;     // [n_ib][n_tiles_total] requantised operand tiles of 2 KiB
+    float *sas;       // [n_ib][n_tiles_total * 16] their per-token scales
+    int *plan;        // [0] macro blocks of this launch, [1 + m] first row block of macro block m
+    int n_ib, nkb, n_mb_max;
+    int blocks_per_macro;   // floor(256 / block_m)
+    int tpb;                // 16-row tile slots per row block in scratch, ceil(block_m / 16)
+    int n_tiles_total;      // n_mb_max * tpb
+    int gps, n_cs;          // 64-column groups per DOWN item, column slabs per macro block
+    int lag;                // macro blocks whose up/gate items precede the first down items of a queue
+    int w_nt;               // weights with non-temporal loads: 1 always, 0 never, -1 for experts with one macro block
+};
+
+#ifndef WIDE_PROBE   // PROBE
+#define WIDE_PROBE 0   // PROBE
+#endif   // PROBE
+#define WPROBE(b) (((WIDE_PROBE) & (b)) != 0)   // PROBE: 1 no up, 2 no down, 4 no y, 8 no reduce, 64 no loads, 128 no mma
+__device__ __forceinline__ int rfl(int v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// A wavefront-uniform pointer the compiler cannot fold into per-lane address arithmetic: added to a 32-bit per-lane
+// offset it gives the "scalar base + vector offset" form of a load, one address register per lane instead of two
+// and no 64-bit vector adds per step.
+template <typename T>
+__device__ __forceinline__ const T *uniform_ptr(const T *ptr)
+{
+    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = (uint32_t)rfl((int)(uint32_t)v), hi = (uint32_t)rfl((int)(uint32_t)(v >> 32));
+    return reinterpret_cast<const T *>(((uint64_t)hi << 32) | lo);
+}
+
+// Direct-to-LDS loads of 16 and 4 bytes per lane from (uniform base + 32-bit per-lane offset).  The empty asm keeps the
+// address addition in the load's own basic block, where instruction selection can fold it into the load.
+template <int AUX>
+__device__ __forceinline__ void dma16_sv(const void *ubase, unsigned voff, void *lds)
+{
+    asm volatile("" : "+v"(voff));
+    const uint8_t *g = uniform_ptr(static_cast<const uint8_t *>(ubase)) + (size_t)voff;
+    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uint32_t)(uintptr_t)lds, 16, 0, AUX);
+}
+template <int AUX>
+__device__ __forceinline__ void dma4_sv(const void *ubase, unsigned voff, void *lds)
+{
+    asm volatile("" : "+v"(voff));
+    const uint8_t *g = uniform_ptr(static_cast<const uint8_t *>(ubase)) + (size_t)voff;
+    __builtin_amdgcn_global_load_lds((gptr_t)(uintptr_t)g, (lptr_t)(uint32_t)(uintptr_t)lds, 4, 0, AUX);
+}
+
+// ---- which row blocks form the macro blocks ------------------------------------------------------------------------
+// One workgroup.  Row block mb leads a macro block when its distance from the first block of its expert's run is a
+// multiple of blocks_per_macro; blocks whose expert id is outside [0, E) lead nothing and belong to nothing.
+__global__ __launch_bounds__(1024) void moe_wide_plan_kernel(const WideParams s)
+{
+    __shared__ int s_last_start[16];
+    __shared__ int s_count[16];
+    __shared__ int s_carry[2];   // run start before this chunk, leaders before this chunk
+    const MoeParams &p = s.p;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int n_live = (p.ntpp[0] + p.block_m - 1) / p.block_m;
+    n_live = n_live < s.n_mb_max ? n_live : s.n_mb_max;
+    if (tid == 0) {
+        s_carry[0] = 0;
+        s_carry[1] = 0;
+    }
+    __syncthreads();
+    for (int base = 0; base < n_live; base += 1024) {
+        const int mb = base + tid;
+        const bool in = mb < n_live;
+        const int e = in ? p.expert_ids[mb] : -1;
+        const int e_prev = (in && mb > 0) ? p.expert_ids[mb - 1] : -2;
+        const bool starts = in && (mb == 0 || e != e_prev);
+        const unsigned long long smask = __ballot(starts);
+        const unsigned long long upto = smask & (~0ull >> (63 - lane));
+        int start = upto ? (base + wave * 64 + 63 - __builtin_clzll(upto)) : -1;
+        if (lane == 63) s_last_start[wave] = start;
+        __syncthreads();
+        if (start < 0) {
+            for (int v = wave - 1; v >= 0 && start < 0; v--) start = s_last_start[v];
+            if (start < 0) start = s_carry[0];
+        }
+        const bool leader = in && e >= 0 && e < p.E && ((mb - start) % s.blocks_per_macro) == 0;
+        const unsigned long long lmask = __ballot(leader);
+        if (lane == 0) s_count[wave] = __builtin_popcountll(lmask);
+        __syncthreads();
+        int pos = s_carry[1] + __builtin_popcountll(lmask & ((1ull << lane) - 1ull));
+        for (int v = 0; v < wave; v++) pos += s_count[v];
+        if (leader) s.plan[1 + pos] = mb;
+        __syncthreads();
+        if (tid == 1023) {
+            int total = pos + (leader ? 1 : 0);
+            s_carry[0] = start;
+            s_carry[1] = total;
+        }
+        __syncthreads();
+    }
+    if (tid == 0) s.plan[0] = s_carry[1];
+}
+
+// One step of a wavefront: the pair's 4 weight tiles x up to 8 token tiles, all from LDS.
+//   acc[k][t] += (A_k x B_t) * row[t] * (k odd ? sc1 : sc0)
+// with row[] a per-token factor in LDS.  Token tile t of the wavefront sits 4 KiB behind tile t - 1 (the other
+// wavefront of the pair owns the tiles in between); only the first nt_w tiles are live.  The product of (k, t) is
+// scaled into its accumulator behind the matrix instruction of (k + 1, t).  issue(t) puts the step's loads between the
+// token tiles, whatever nt_w is.
+template <typename Issue>
+__device__ __forceinline__ void wide_step(const uint8_t *a_tiles, const uint8_t *b_tiles, const float *row, float sc0,
+                                          float sc1, v4f (&acc)[4][8], int frag_lo, int frag_hi, int nt_w, Issue issue)
+{
+    auto read_tile = [&](const uint8_t *tile) -> v8i {
+        return cat(*reinterpret_cast<const v4i *>(tile + frag_lo), *reinterpret_cast<const v4i *>(tile + frag_hi));
+    };
+    v8i a[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) a[k] = read_tile(a_tiles + k * 2048);
+    v8i b = read_tile(b_tiles);
+    float f = row[0];
+#pragma unroll
+    for (int t = 0; t < 8; t++) {
+        issue(t);
+        v8i b_next = b;
+        float f_next = f;
+        if (t + 1 < 8) {
+            b_next = read_tile(b_tiles + (t + 1) * 4096);
+            // per-token factors of tile tt sit at (tt & 7) * 32 + (tt >> 3) * 16; tt = 2 t + g, g folded into `row`
+            f_next = row[(t + 1) < 4 ? (t + 1) * 64 : (t + 1 - 4) * 64 + 16];
+        }
+        if (t < nt_w && !WPROBE(128)) {
+            const float p0 = f * sc0, p1 = f * sc1;
+            v4f prev;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const v4f cur = mfma_fp8(a[k], b);
+                __builtin_amdgcn_sched_barrier(0);
+                if (k > 0) {
+                    acc[k - 1][t] += prev * (((k - 1) & 1) ? p1 : p0);
+                    asm volatile("" : "+v"(acc[k - 1][t]));   // the multiply-adds stay behind this matrix instruction
+                }
+                prev = cur;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            acc[3][t] += prev * p1;
+            asm volatile("" : "+v"(acc[3][t]));
+        }
+        b = b_next;
+        f = f_next;
+    }
+}
+
+__global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
+{
+    constexpr int THREADS = 512;
+    // [2 stages][4 pairs][4 tiles] weight ring | [2 stages][16] token tiles (UP, streamed DOWN) or the requantised
+    // tiles [n_ib][16] of a resident DOWN item in the same place
+    extern __shared__ __attribute__((aligned(1024))) uint8_t lds_dyn[];
+    __shared__ float s_xs[2][kWRows];        // per-token factors of a ring stage, tile tt at (tt & 7) * 32 + (tt >> 3) * 16
+    __shared__ float s_ws[2][kWMaxKb];
+    __shared__ float s_amax[4][kWRows];
+    __shared__ float s_w2s[kWMaxW2s];
+    __shared__ int s_tok[kWRows];            // UP: token of each row (-1: none); DOWN: slot of each row (-1: none)
+    __shared__ float s_tw[kWRows];
+    __shared__ int s_last[4];
+    __shared__ int s_item[2];
+
+    const MoeParams &p = s.p;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = rfl(tid >> 6);
+    const int w = wave & 3, g = wave >> 2;
+    const int n = lane & 15;
+    const int q = lane >> 4;
+    const int K = p.K, I = p.N >> 1;
+    const int n_ib = s.n_ib, nkb = s.nkb;
+    const int epoch = (int)((unsigned)rfl(s.ctl->epoch) + 1u);
+    uint8_t *a_ring = lds_dyn;
+    uint8_t *xbuf = lds_dyn + 2 * kWStageA;
+
+    int n_live = (rfl(p.ntpp[0]) + p.block_m - 1) / p.block_m;
+    n_live = n_live < s.n_mb_max ? n_live : s.n_mb_max;
+    const int n_macro = rfl(s.plan[0]);
+    const int per_q = (n_macro + 7) >> 3;
+    const int per_up = n_ib, per_down = s.n_cs;
+
+    // operand fragment of lane (n, q): chunks q and q+4 of row n; chunk c of row r sits at position c ^ ((r >> 1) & 7)
+    const int f_n = (n >> 1) & 7;
+    const int frag_lo = n * 128 + 16 * (q ^ f_n);
+    const int frag_hi = n * 128 + 16 * ((q ^ f_n) ^ 4);
+    // direct-to-LDS load h of a tile: lane l fills position l & 7 of row 8h + l / 8
+    const int ld_row = lane >> 3;
+    unsigned ld_chunk[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) ld_chunk[h] = 16u * ((lane & 7) ^ (((8 * h + ld_row) >> 1) & 7));
+    // per-token factors of this lane's token in tile g (later tiles: see wide_step)
+    const int row_off = g * 32 + n;
+
+    v4f acc[4][8];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int a = 0; a < 4; a++)
+#pragma unroll
+            for (int t = 0; t < 8; t++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+    };
+
+    // Rows of macro block m: row blocks mb0 .. mb0 + nb - 1 of expert e, sorted rows row0 .. row0 + n_rows - 1.
+    struct Macro {
+        int mb0, e, row0, n_rows;
+        bool lone;   // the expert has no other macro block
+    };
+    auto macro_of = [&](int m) {
+        Macro mc;
+        mc.mb0 = rfl(s.plan[1 + m]);
+        mc.e = rfl(p.expert_ids[mc.mb0]);
+        int nb = 1;
+        while (nb < s.blocks_per_macro && mc.mb0 + nb < n_live && rfl(p.expert_ids[mc.mb0 + nb]) == mc.e) nb++;
+        mc.row0 = mc.mb0 * p.block_m;
+        mc.n_rows = nb * p.block_m;
+        if (mc.row0 + mc.n_rows > p.sorted_num) mc.n_rows = p.sorted_num - mc.row0;
+        const bool left = mc.mb0 > 0 && rfl(p.expert_ids[mc.mb0 - 1]) == mc.e;
+        const bool right = mc.mb0 + nb < n_live && rfl(p.expert_ids[mc.mb0 + nb]) == mc.e;
+        mc.lone = s.w_nt >= 0 ? s.w_nt != 0 : (!left && !right);
+        return mc;
+    };
+    // Routing of the block's rows into LDS; returns the number of 16-row tiles up to the last valid row.
+    auto load_rows = [&](const Macro &mc, bool for_down, int cs) {
+        if (tid < kWRows) {
+            int id = -1;
+            if (tid < mc.n_rows) id = p.sorted_ids[mc.row0 + tid];
+            const int tk = id / p.top_k;
+            const bool ok = id >= 0 && tk < p.M;
+            if (!for_down) {
+                s_tok[tid] = ok ? (WPROBE(16) ? 0 : tk) : -1;
+            } else {
+                s_tok[tid] = ok ? id : -1;
+                s_tw[tid] = ok ? p.topk_w[id] * p.scaling : 0.f;
+                if (ok && cs == 0) s.live[id] = epoch;
+            }
+            const unsigned long long okm = __ballot(ok);
+            if (lane == 0) s_last[wave] = okm ? wave * 64 + 63 - __builtin_clzll(okm) : -1;
+        }
+    };
+    auto tiles_of = [&]() {
+        int last = s_last[0];
+#pragma unroll
+        for (int v = 1; v < 4; v++) last = s_last[v] > last ? s_last[v] : last;
+        return rfl((last >> 4) + 1);   // 0 when no row is valid
+    };
+
+    // ---- UP item: slice ib of macro block m -> requantised operand tiles + scales in scratch, then the unit's flag --
+    auto up_item = [&](int m, int ib) {
+        const Macro mc = macro_of(m);
+        load_rows(mc, false, 0);
+        {
+            // this slice's gate (row 2*ib) and up (row 2*ib+1) scale rows
+            const float *ws_rows = p.w_scale + ((size_t)mc.e * (p.N >> 7) + 2 * ib) * nkb;
+            for (int i = tid; i < 2 * nkb; i += THREADS) s_ws[i >= nkb][i >= nkb ? i - nkb : i] = ws_rows[i];
+        }
+        __syncthreads();
+        const int n_tiles = tiles_of();
+        const int nt_w = n_tiles > g ? (n_tiles - g + 1) >> 1 : 0;
+        const int unit = mc.mb0 * n_ib + ib;
+        if (n_tiles > 0) {
+            // token-tile gather: wavefront v loads tiles v and v + 8
+            unsigned x_off[2][2], xs_off;
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const int tk = s_tok[(wave + 8 * j) * 16 + 8 * h + ld_row];
+                    x_off[j][h] = (unsigned)(tk < 0 ? 0 : tk) * (unsigned)K + ld_chunk[h];
+                }
+            {
+                const int tk = s_tok[(wave + 8 * ((lane >> 4) & 1)) * 16 + n];
+                xs_off = (unsigned)(tk < 0 ? 0 : tk) * (unsigned)nkb;
+            }
+            // Weight rows of the pair: tile a = (32-row group a / 2, gate | up a % 2); matrix row r of the tile is slab
+            // row group * 32 + (r / 8) * 16 + r % 8 (+ 8 for up), so load h of a tile covers slab rows ... + 16 h +
+            // lane / 8.  Wavefront (w, g) loads tiles 2g and 2g + 1 of pair w.
+            unsigned w_off[2][2];
+#pragma unroll
+            for (int up = 0; up < 2; up++)
+#pragma unroll
+                for (int h = 0; h < 2; h++)
+                    w_off[up][h] =
+                        (unsigned)((ib * 256 + w * 64 + g * 32 + ld_row + h * 16 + 8 * up) * p.w_rs) + ld_chunk[h];
+            const uint8_t *wexp = p.w + (size_t)(WPROBE(32) ? mc.e & 7 : mc.e) * p.N * K;
+            const bool nt = mc.lone;
+            // operation i of a step: 4 weight tile halves, 4 token tile halves, the token scales
+            auto issue_op = [&](int kb, int stage, int i) {
+                if (WPROBE(64)) return;   // PROBE
+                if (i < 4) {
+                    const int up = i >> 1, h = i & 1;
+                    const uint8_t *src = wexp + (size_t)kb * p.w_ks;
+                    uint8_t *dst = a_ring + stage * kWStageA + w * 8192 + (2 * g + up) * 2048 + h * 1024;
+                    if (nt) dma16_sv<2>(src, w_off[up][h], dst);
+                    else dma16_sv<0>(src, w_off[up][h], dst);
+                } else if (i < 8) {
+                    const int j = (i - 4) >> 1, h = i & 1;
+                    if (wave + 8 * j < n_tiles)
+                        dma16_sv<0>(p.x + (size_t)kb * 128, x_off[j][h],
+                                    xbuf + stage * kWStageX + (wave + 8 * j) * 2048 + h * 1024);
+                } else {
+                    if (lane < 32) dma4_sv<0>(p.x_scale + kb, xs_off * 4u, &s_xs[stage][wave * 32]);
+                }
+            };
+            clear_acc();
+#if (WIDE_PROBE & 0x300)   // PROBE: loads only, 2 or 3 steps in flight (LDS contents are garbage)
+            {   // PROBE
+                constexpr int D = (WIDE_PROBE & 0x200) ? 3 : 2;   // PROBE
+                for (int d = 0; d < D; d++)   // PROBE
+                    for (int i = 0; i < 9; i++) issue_op(d < nkb ? d : nkb - 1, d & 1, i);   // PROBE
+                for (int kb = 0; kb < nkb; kb++) {   // PROBE
+                    wait_vmcnt<9 * (D - 1)>();   // PROBE
+                    lds_barrier();   // PROBE
+                    for (int i = 0; i < 9; i++) issue_op(kb + D < nkb ? kb + D : nkb - 1, kb & 1, i);   // PROBE
+                }   // PROBE
+                wait_vmcnt<0>();   // PROBE
+            }   // PROBE
+            if (false)   // PROBE
+#endif   // PROBE
+            {
+#pragma unroll
+            for (int i = 0; i < 9; i++) issue_op(0, 0, i);
+            wait_vmcnt<0>();
+            }
+            for (int kb0 = 0; kb0 < nkb && !(WIDE_PROBE & 0x300); kb0 += 2) {
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const int kb = kb0 + h;
+                    if (kb < nkb) {
+                        lds_barrier();
+                        wide_step(a_ring + h * kWStageA + w * 8192, xbuf + h * kWStageX + g * 2048, &s_xs[h][row_off],
+                                  s_ws[0][kb], s_ws[1][kb], acc, frag_lo, frag_hi, nt_w, [&](int t) {
+                                      if (kb + 1 < nkb) {
+                                          // 9 loads over the first four token tiles: 3, 2, 2, 2
+                                          if (t == 0) {
+                                              issue_op(kb + 1, h ^ 1, 0);
+                                              issue_op(kb + 1, h ^ 1, 4);
+                                              issue_op(kb + 1, h ^ 1, 8);
+                                          } else if (t < 4) {
+                                              issue_op(kb + 1, h ^ 1, t);
+                                              issue_op(kb + 1, h ^ 1, t + 4);
+                                          }
+                                      }
+                                  });
+                        wait_vmcnt<0>();
+                    }
+                }
+            }
+
+            // SwiGLU, per-token amax over the slice's 128 columns, FP8 requant into operand tiles
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                if (t < nt_w) {
+                    float mx = 0.f;
+#pragma unroll
+                    for (int pr = 0; pr < 2; pr++)
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const float a = swiglu_bf16(acc[2 * pr][t][j], acc[2 * pr + 1][t][j]);
+                            acc[2 * pr][t][j] = a;
+                            mx = fmaxf(mx, fabsf(a));
+                        }
+                    mx = fmaxf(mx, __shfl_xor(mx, 16));
+                    mx = fmaxf(mx, __shfl_xor(mx, 32));
+                    if (q == 0) s_amax[w][(2 * t + g) * 16 + n] = mx;
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                if (t < nt_w) {
+                    const int tt = 2 * t + g;
+                    float mx = kAmaxFloor;
+#pragma unroll
+                    for (int wv = 0; wv < 4; wv++) mx = fmaxf(mx, s_amax[wv][tt * 16 + n]);
+                    const float s_a = mx / kFp8Max;
+                    const size_t gt = (size_t)ib * s.n_tiles_total + (size_t)mc.mb0 * s.tpb + tt;
+                    uint8_t *tile = s.aqs + gt * 2048;
+#pragma unroll
+                    for (int pr = 0; pr < 2; pr++) {
+                        const uint32_t packed =
+                            pack_fp8x4(clamp_fp8(acc[2 * pr][t][0] / s_a), clamp_fp8(acc[2 * pr][t][1] / s_a),
+                                       clamp_fp8(acc[2 * pr][t][2] / s_a), clamp_fp8(acc[2 * pr][t][3] / s_a));
+                        // columns w*32 + pr*16 + 4q .. +3 of token n: chunk w*2 + pr of the row, bytes 4q .. 4q+3 in it
+                        stg32_agent(tile + n * 128 + 16 * ((w * 2 + pr) ^ f_n) + 4 * q, packed);
+                    }
+                    if (w == 0 && q == 0) stg32_agent(&s.sas[gt * 16 + n], __builtin_bit_cast(uint32_t, s_a));
+                }
+            }
+            wait_vmcnt<0>();
+        }
+        __syncthreads();
+        if (tid == 0) store_agent(&s.flag[unit], epoch);
+    };
+
+    // ---- DOWN item: column groups [cs * gps, (cs + 1) * gps) of macro block m, all slices ---------------------------
+    // 64 output columns per pair of wavefronts and step.  Pair w takes the slab's groups w, w + 4, ...; its two
+    // wavefronts split the token tiles as above and each loads two of the four w2 tiles of a step.  Matrix row r of tile
+    // k is output column c0 + 16 (r / 4) + 4 k + r % 4, so lane (n, q) collects columns c0 + 16 q .. c0 + 16 q + 15 of
+    // token n over the four tiles.  Load h of a tile: rows 8h + lane / 8.
+    auto down_item = [&](int m, int cs, auto resident_c) {
+        constexpr bool RESIDENT = decltype(resident_c)::value;
+        const Macro mc = macro_of(m);
+        load_rows(mc, true, cs);
+        for (int i = tid; i < (K >> 7) * n_ib; i += THREADS) s_w2s[i] = p.w2_scale[(size_t)mc.e * (K >> 7) * n_ib + i];
+        const bool nt = mc.lone;
+
+        const int n_groups = K >> 6;
+        const int g0 = cs * s.gps;
+        const int g1 = g0 + s.gps < n_groups ? g0 + s.gps : n_groups;
+        const int span = g1 - g0;
+        int my_groups = (span - w + 3) >> 2;                      // the slab's groups w, w + 4, ... (none: 0)
+        my_groups = my_groups > 0 ? my_groups : 0;
+        const int n_steps = ((span + 3) >> 2) * n_ib;             // (group, slice) steps of the longest pair, slice-minor
+        const uint8_t *w2exp = p.w2 + (size_t)mc.e * K * I;
+        unsigned w2_off[2][2];
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                w2_off[kk][h] =
+                    (unsigned)((16 * (lane >> 5) + (ld_row & 3) + 32 * h + 4 * (2 * g + kk)) * p.w2_rs) + ld_chunk[h];
+        int lg = 0, lib = 0;   // (group index, slice) of the next step to load
+        auto group_of = [&](int i) {   // i-th group of this pair, clamped into the slab for loads past its end
+            int grp = g0 + w + 4 * (i < my_groups ? i : my_groups - 1);
+            grp = grp < g0 ? g0 : grp;
+            return grp < g1 ? grp : g1 - 1;
+        };
+        const size_t tile0 = (size_t)mc.mb0 * s.tpb;
+        int n_tiles = 0;
+        // operation i of the step (lg, lib) into ring stage `stage`: 4 w2 tile halves; streamed: 4 requantised tile
+        // halves of slice lib and their scales
+        auto issue_op = [&](int stage, int i) {
+            if (WPROBE(64)) return;   // PROBE
+            if (i < 4) {
+                const int kk = i >> 1, h = i & 1;
+                const int c0 = group_of(lg) << 6;
+                const uint8_t *src = w2exp + (size_t)c0 * p.w2_rs + (size_t)lib * p.w2_ks;
+                uint8_t *dst = a_ring + stage * kWStageA + w * 8192 + (2 * g + kk) * 2048 + h * 1024;
+                if (nt) dma16_sv<2>(src, w2_off[kk][h], dst);
+                else dma16_sv<0>(src, w2_off[kk][h], dst);
+            } else if (!RESIDENT) {
+                if (i < 8) {
+                    const int j = (i - 4) >> 1, h = i & 1;
+                    if (wave + 8 * j < n_tiles)
+                        dma16_sv<16>(s.aqs + ((size_t)lib * s.n_tiles_total + tile0 + wave + 8 * j) * 2048 + h * 1024,
+                                     (unsigned)(lane * 16), xbuf + stage * kWStageX + (wave + 8 * j) * 2048 + h * 1024);
+                } else if (lane < 32) {
+                    const int tt = wave + 8 * ((lane >> 4) & 1);
+                    dma4_sv<16>(s.sas + ((size_t)lib * s.n_tiles_total + tile0) * 16,
+                                (unsigned)((tt < n_tiles ? tt : 0) * 16 + n) * 4u, &s_xs[stage][wave * 32]);
+                }
+            }
+        };
+        auto advance = [&]() {
+            lib++;
+            if (lib == n_ib) {
+                lib = 0;
+                lg++;
+            }
+        };
+        // the weights do not depend on the up/gate phase: the first step's go out before the wait
+#pragma unroll
+        for (int i = 0; i < 4; i++) issue_op(0, i);
+        if (wave == 0) spin_all_ge(&s.flag[mc.mb0 * n_ib], n_ib, epoch, s.ctl);
+        __syncthreads();
+        n_tiles = tiles_of();
+        const int nt_w = n_tiles > g ? (n_tiles - g + 1) >> 1 : 0;
+        if (RESIDENT) {
+            // the requantised tiles of all slices and their scales come from scratch into LDS: [slice][tile]
+            for (int i = wave; i < n_ib * kWTiles; i += 8) {
+                const int ib = i >> 4, tt = i & 15;
+                if (tt < n_tiles) {
+                    const uint8_t *src = s.aqs + ((size_t)ib * s.n_tiles_total + tile0 + tt) * 2048;
+                    dma16_sv<16>(src, (unsigned)(lane * 16), xbuf + i * 2048);
+                    dma16_sv<16>(src + 1024, (unsigned)(lane * 16), xbuf + i * 2048 + 1024);
+                }
+            }
+            for (int i = tid; i < n_ib * kWRows; i += THREADS) {
+                const int ib = i >> 8, r = i & 255;
+                const int tt = r >> 4;
+                if (tt < n_tiles) {
+                    const int bits = load_agent(reinterpret_cast<const int *>(
+                        &s.sas[((size_t)ib * s.n_tiles_total + tile0 + tt) * 16 + (r & 15)]));
+                    s_xs[ib][(tt & 7) * 32 + (tt >> 3) * 16 + (r & 15)] = __builtin_bit_cast(float, bits);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 4; i < 9; i++) issue_op(0, i);
+        }
+        advance();
+        wait_vmcnt<0>();
+        clear_acc();
+        int cg = 0, cib = 0;
+        for (int s0 = 0; s0 < n_steps; s0 += 2) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                if (s0 + h < n_steps) {
+                    lds_barrier();
+                    const int c0 = group_of(cg) << 6;
+                    const float ws2 = s_w2s[(c0 >> 7) * n_ib + cib];
+                    const bool more = s0 + h + 1 < n_steps;
+                    const uint8_t *b_tiles = RESIDENT ? xbuf + cib * kWStageX + g * 2048 : xbuf + h * kWStageX + g * 2048;
+                    const float *row = RESIDENT ? &s_xs[cib][row_off] : &s_xs[h][row_off];
+                    wide_step(a_ring + h * kWStageA + w * 8192, b_tiles, row, ws2, ws2, acc, frag_lo, frag_hi, nt_w,
+                              [&](int t) {
+                                  if (more) {
+                                      if (RESIDENT) {
+                                          if (t < 4) issue_op(h ^ 1, t);
+                                      } else if (t == 0) {
+                                          issue_op(h ^ 1, 0);
+                                          issue_op(h ^ 1, 4);
+                                          issue_op(h ^ 1, 8);
+                                      } else if (t < 4) {
+                                          issue_op(h ^ 1, t);
+                                          issue_op(h ^ 1, t + 4);
+                                      }
+                                  }
+                              });
+                    if (more) advance();
+                    // the next step's loads have landed before any result store is issued: the stores are then only
+                    // waited for a whole step later
+                    wait_vmcnt<0>();
+                    cib++;
+                    if (cib == n_ib) {
+#pragma unroll
+                        for (int t = 0; t < 8; t++) {
+                            if (t < nt_w) {
+                                const int r = (2 * t + g) * 16 + n;
+                                const int slot = s_tok[r];
+                                if (slot >= 0 && cg < my_groups && !WPROBE(4)) {
+                                    const float tw = s_tw[r];
+                                    uint16_t *yp = s.y + (size_t)slot * K + c0 + 16 * q;
+#pragma unroll
+                                    for (int half = 0; half < 2; half++) {
+                                        const v4f lo = acc[2 * half][t] * tw, hi = acc[2 * half + 1][t] * tw;
+                                        v4i o;
+                                        o.x = (int)pack_bf16x2(lo[0], lo[1]);
+                                        o.y = (int)pack_bf16x2(lo[2], lo[3]);
+                                        o.z = (int)pack_bf16x2(hi[0], hi[1]);
+                                        o.w = (int)pack_bf16x2(hi[2], hi[3]);
+                                        *reinterpret_cast<v4i *>(yp + 8 * half) = o;
+                                    }
+                                }
+#pragma unroll
+                                for (int a = 0; a < 4; a++) acc[a][t] = (v4f){0.f, 0.f, 0.f, 0.f};
+                            }
+                        }
+                        cib = 0;
+                        cg++;
+                    }
+                }
+            }
+        }
+        wait_vmcnt<0>();
+    };
+
+    // ---- item loop ------------------------------------------------------------------------------------------------
+    // Queue qq holds macro blocks [qq * per_q, ...) as items: the up/gate items of `lag` blocks first, then alternately
+    // the up/gate items of block lag + r and the down items of block r, at the end the down items of the last `lag`
+    // blocks.  A down item waits for the flags of its block's up/gate items, which are EARLIER in the same queue:
+    // whoever took them is running and waits for nothing later, so the queues drain with any number of resident
+    // workgroups.  A workgroup that finds its queue empty moves on to the next one.
+    auto blocks_of = [&](int qq) {
+        const int left = n_macro - qq * per_q;
+        return left < 0 ? 0 : (left < per_q ? left : per_q);
+    };
+    int qq = blockIdx.x & 7, visited = 0;   // state of thread 0
+    while (true) {
+        if (tid == 0) {
+            int it = -1;
+            while (visited < 8) {
+                const int nb = blocks_of(qq);
+                const int idx = nb > 0 ? __hip_atomic_fetch_add(&s.ctl->tile_head[qq], 1, __ATOMIC_RELAXED,
+                                                                __HIP_MEMORY_SCOPE_AGENT)
+                                       : 0;
+                if (idx < nb * (per_up + per_down)) {
+                    it = idx;
+                    break;
+                }
+                qq = (qq + 1) & 7;
+                visited++;
+            }
+            s_item[0] = it;
+            s_item[1] = qq;
+        }
+        __syncthreads();
+        const int item = rfl(s_item[0]);
+        const int qi = rfl(s_item[1]);
+        if (item < 0) break;
+        const int nb = blocks_of(qi);
+        const int lag = s.lag < nb ? s.lag : nb;
+        const int head_items = lag * per_up, mid_items = (nb - lag) * (per_up + per_down);
+        int up = -1, down = -1;
+        if (item < head_items) {
+            up = item;
+        } else if (item < head_items + mid_items) {
+            const int i = item - head_items;
+            const int round = i / (per_up + per_down);
+            const int off = i - round * (per_up + per_down);
+            if (off < per_up)
+                up = (lag + round) * per_up + off;
+            else
+                down = round * per_down + (off - per_up);
+        } else {
+            down = (nb - lag) * per_down + (item - head_items - mid_items);
+        }
+        if (up >= 0) {
+            if (!WPROBE(1)) up_item(qi * per_q + up / per_up, up % per_up);
+            else if (tid == 0) store_agent(&s.flag[rfl(s.plan[1 + qi * per_q + up / per_up]) * n_ib + up % per_up], epoch);   // PROBE
+        } else if (WPROBE(2)) {   // PROBE
+        } else if (n_ib <= kWResidentIb) {
+            down_item(qi * per_q + down / per_down, down % per_down, std::true_type());
+        } else {
+            down_item(qi * per_q + down / per_down, down % per_down, std::false_type());
+        }
+        __syncthreads();   // everybody is done with the item's LDS tables and rings before the next item refills them
+    }
+    if (tid == 0) {
+        const int left = __hip_atomic_fetch_add(&s.ctl->tile_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (left == (int)gridDim.x - 1) {
+            for (int i = 0; i < 8; i++) store_agent(&s.ctl->tile_head[i], 0);
+            store_agent(&s.ctl->tile_done, 0);
+        }
+    }
+}
+
+size_t align_up(size_t v) { return (v + 255) & ~(size_t)255; }
+
+hipError_t allow_dynamic_lds()
+{
+    static std::mutex mu;
+    static bool done[64];
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) return err;
+    std::lock_guard<std::mutex> lock(mu);
+    if (dev >= 0 && dev < 64 && done[dev]) return hipSuccess;
+    err = hipFuncSetAttribute(reinterpret_cast<const void *>(moe_wide_kernel),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kWDynLds);
+    if (err == hipSuccess && dev >= 0 && dev < 64) done[dev] = true;
+    return err;
+}
+
+// 64-column groups per DOWN item: about 16 ring steps (a step is four groups x one slice), a multiple of 4 so that
+// every pair of wavefronts gets the same number of groups
+int groups_per_item(int n_ib)
+{
+    const int e = tunable(kTunTileGps, 0);
+    if (e > 0) return (e + 3) / 4 * 4;
+    return 4 * ((16 + n_ib - 1) / n_ib);
+}
+
+}  // namespace
+
+bool wide_supported(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
+{
+    (void)E;
+    const int n_ib = N / 256;
+    const int64_t n_mb = ((int64_t)sorted_num + block_m - 1) / block_m;
+    return block_m > 32 && K <= 128 * kWMaxKb && (K / 128) * n_ib <= kWMaxW2s && (int64_t)M * top_k <= kMaxSlots &&
+           n_mb * n_ib <= kMaxUnits && (int64_t)N * K < ((int64_t)1 << 31) && (int64_t)M * K < ((int64_t)1 << 32);
+}
+
+size_t wide_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
+{
+    (void)E;
+    const size_t n_mb = ((size_t)sorted_num + block_m - 1) / block_m;
+    const size_t tiles = n_mb * ((block_m + 15) / 16);
+    return align_up(kPrefixBytes) + align_up((size_t)M * top_k * K * sizeof(uint16_t)) +
+           align_up((size_t)(N / 256) * tiles * 2048) + align_up((size_t)(N / 256) * tiles * 16 * sizeof(float)) +
+           align_up((n_mb + 1) * sizeof(int));
+}
+
+hipError_t launch_wide(const MoeParams &p, void *workspace, hipStream_t stream)
+{
+    uint8_t *ws = static_cast<uint8_t *>(workspace);
+    WideParams s;
+    s.p = p;
+    s.n_ib = p.N / 256;
+    s.nkb = p.K / 128;
+    s.n_mb_max = (p.sorted_num + p.block_m - 1) / p.block_m;
+    s.blocks_per_macro = kWRows / p.block_m;
+    s.tpb = (p.block_m + 15) / 16;
+    s.n_tiles_total = s.n_mb_max * s.tpb;
+    size_t off = align_up(kPrefixBytes);
+    s.ctl = reinterpret_cast<StreamCtl *>(ws);
+    s.flag = reinterpret_cast<int *>(ws + kOffFlag);
+    s.live = reinterpret_cast<int *>(ws + kOffLive);
+    s.y = reinterpret_cast<uint16_t *>(ws + off);
+    off += align_up((size_t)p.M * p.top_k * p.K * sizeof(uint16_t));
+    s.aqs = ws + off;
+    off += align_up((size_t)s.n_ib * s.n_tiles_total * 2048);
+    s.sas = reinterpret_cast<float *>(ws + off);
+    off += align_up((size_t)s.n_ib * s.n_tiles_total * 16 * sizeof(float));
+    s.plan = reinterpret_cast<int *>(ws + off);
+    s.gps = groups_per_item(s.n_ib);
+    s.n_cs = ((p.K >> 6) + s.gps - 1) / s.gps;
+    s.lag = tunable(kTunTileLag, 32);
+    s.w_nt = tunable(kTunTileNt, -1);
+    if (s.lag < 1) s.lag = 1;
+    hipError_t err = allow_dynamic_lds();
+    if (err != hipSuccess) return err;
+    hipLaunchKernelGGL(moe_wide_plan_kernel, dim3(1), dim3(1024), 0, stream, s);
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            return 256;
+        return n;
+    }();
+    const int64_t items = (int64_t)s.n_mb_max * (s.n_ib + s.n_cs);
+    int grid = tunable(kTunTileGrid, cus);
+    if (grid > items) grid = (int)((items + 7) / 8 * 8);
+    if (grid < 8) grid = 8;
+    hipLaunchKernelGGL(moe_wide_kernel, dim3((unsigned)grid), dim3(512), kWDynLds, stream, s);
+    err = hipGetLastError();
+    if (err != hipSuccess) return err;
+    if (WPROBE(8)) return hipSuccess;   // PROBE
+    RowsReduce r;
+    r.p = p;
+    r.ctl = s.ctl;
+    r.live = s.live;
+    r.y = s.y;
+    return launch_rows_reduce(r, stream);
+}
+
+}  // namespace alpha_moe

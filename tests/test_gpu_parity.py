@@ -91,11 +91,23 @@ def test_store_variant_overwrites_whatever_out_held(c1, knobs):
     P.topk_weights = saved
 
 
+def test_nine_slices_row_blocks_above_32():
+    """Nine 128-column slices are more than the tile kernel takes: the wide kernel streams any number of them, whatever
+    (block_n, warp_n) asks for."""
+    shape = Shape("s9", E=6, top_k=2, K=256, I=1152, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0)
+    W = make_weights(shape, device=DEV, seed=5)
+    P = make_problem(W, 150, seed=5)
+    ref = oracle_out(P)
+    for knobs in ((128, 64, 4, 2), (64, 32, 8, 3)):
+        print(f"case nine slices knobs {knobs}", flush=True)
+        assert_parity(run_op(P, *knobs, via="c_abi"), ref, f"nine slices {knobs}")
+
+
 def test_store_variant_fallback_kernel():
-    """Nine 128-column slices are more than the tile kernel takes: the fallback kernel serves the call, and its store
+    """129 K blocks are more than the tile and wide kernels take: the fallback kernel serves the call, and its store
     variant overwrites too."""
     from alpha_moe_python.workloads import Shape
-    shape = Shape("fb", E=6, top_k=2, K=256, I=1152, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0)
+    shape = Shape("fb", E=6, top_k=2, K=16512, I=128, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0)
     W = make_weights(shape, device=DEV, seed=5)
     P = make_problem(W, 150, seed=5)
     ref = oracle_out(P)
@@ -742,7 +754,7 @@ def test_prepacked_weights_give_the_same_bits(c1, ds_weights, q3_weights):
         del packed
     # shapes only the fallback kernel takes are refused for pre-packed weights
     import alpha_moe
-    shape = Shape("fb", E=2, top_k=1, K=128, I=1152, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0)
+    shape = Shape("fb", E=2, top_k=1, K=16512, I=128, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0)
     Wf = make_weights(shape, device=DEV, seed=5)
     Pf = make_problem(Wf, 8, seed=5)
     with pytest.raises(AssertionError):
