@@ -38,6 +38,10 @@ c_abi.alpha_moe_fused_moe_w8a8_up_down_prepacked.restype = ctypes.c_int
 c_abi.alpha_moe_fused_moe_w8a8_up_down_prepacked.argtypes = (
     [ctypes.c_void_p] * 11 + [ctypes.c_int] * 10 + [ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
                                                    ctypes.c_void_p])
+c_abi.alpha_moe_static_scratch_check.restype = ctypes.c_int
+c_abi.alpha_moe_static_scratch_check.argtypes = [ctypes.c_void_p]
+c_abi.alpha_moe_static_scratch_reset.restype = ctypes.c_int
+c_abi.alpha_moe_static_scratch_reset.argtypes = [ctypes.c_void_p]
 c_abi.alpha_moe_set_tunable.restype = ctypes.c_int
 c_abi.alpha_moe_set_tunable.argtypes = [ctypes.c_char_p, ctypes.c_int, ctypes.c_int]
 c_abi.alpha_moe_workspace_check.restype = ctypes.c_int

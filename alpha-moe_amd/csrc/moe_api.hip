@@ -155,9 +155,9 @@ int run_fused_moe(const uint8_t *x, const float *x_scale, const uint8_t *w, cons
     if (path == kStream) {
         err = launch_stream(p, warp_n, stages, workspace, hs);
     } else if (path == kWide) {
-        err = launch_wide(p, workspace, hs);
+        err = launch_wide(p, stages, workspace, hs);
     } else if (path == kTile) {
-        err = launch_tile(p, workspace, hs);
+        err = launch_tile(p, stages, workspace, hs);
     } else {
         // the fallback kernel reads the operator's own layout only
         if (prepacked) return ALPHA_MOE_ERR_SHAPE;
@@ -265,6 +265,31 @@ extern "C" int alpha_moe_fused_moe_w8a8_up_down_static(const uint8_t *x, const f
                          warp_n, stages, scaling_factor, ptr, ALPHA_MOE_STATIC_SCRATCH_BYTES, stream, 0);
 }
 
+namespace {
+// clears `words` ints (a fill kernel: unlike a memset node it may be recorded into a HIP graph)
+__global__ void zero_words_kernel(int *dst, size_t words)
+{
+    for (size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x; i < words; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = 0;
+}
+}  // namespace
+
+extern "C" int alpha_moe_static_scratch_check(void *stream)
+{
+    void *ptr = static_scratch_of_current_device();
+    if (!ptr) return ALPHA_MOE_ERR_LAUNCH;
+    return alpha_moe_workspace_check(ptr, stream);
+}
+
+extern "C" int alpha_moe_static_scratch_reset(void *stream)
+{
+    void *ptr = static_scratch_of_current_device();
+    if (!ptr) return ALPHA_MOE_ERR_LAUNCH;
+    hipLaunchKernelGGL(zero_words_kernel, dim3(64), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<int *>(ptr), alpha_moe_workspace_zero_bytes() / sizeof(int));
+    return hipGetLastError() == hipSuccess ? ALPHA_MOE_OK : ALPHA_MOE_ERR_LAUNCH;
+}
+
 extern "C" int alpha_moe_workspace_check(const void *workspace, void *stream)
 {
     if (!workspace) return ALPHA_MOE_ERR_NULL_POINTER;
@@ -300,4 +325,4 @@ extern "C" const char *alpha_moe_status_string(int status)
     }
 }
 
-extern "C" const char *alpha_moe_version(void) { return "0.3"; }
+extern "C" const char *alpha_moe_version(void) { return "0.4"; }

@@ -16,6 +16,7 @@
 #include <stdint.h>
 
 #include "../../include/alpha_moe_hip.h"
+#include "alpha_moe_tuning.h"
 
 namespace alpha_moe {
 
@@ -227,8 +228,9 @@ __device__ __forceinline__ bool reached(int a, int b) { return (int)((unsigned)a
 
 // A whole wavefront, `count` <= 64 consecutive flags, one per lane: every poll is ONE load, so the wait costs one round
 // trip however many flags there are.
-// `also`: a counter that other workgroups are (or will be) waiting on; an expiry adds kExpiredBit to it, so that they
-// stop waiting and learn about the expiry from the very word they poll.
+// `also`: a counter that other workgroups are (or will be) waiting on; an expiry sets kExpiredBit in it (an OR: several
+// wavefronts of a workgroup may expire together and must not cancel each other), so that they stop waiting and learn
+// about the expiry from the very word they poll.
 constexpr int kExpiredBit = 1 << 30;
 __device__ __noinline__ inline void spin_all_ge(const int *addr, int count, int target, StreamCtl *ctl,
                                                 int *also = nullptr)
@@ -242,7 +244,7 @@ __device__ __noinline__ inline void spin_all_ge(const int *addr, int count, int 
     }
     if (lane == 0) {
         store_agent(&ctl->error, 1);
-        if (also) __hip_atomic_fetch_add(also, kExpiredBit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (also) __hip_atomic_fetch_or(also, kExpiredBit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -287,13 +289,13 @@ hipError_t launch_stream(const MoeParams &p, int warp_n, int stages, void *works
 // one workgroup, per-slot bf16 result rows reduced by a second kernel.
 bool tile_supported(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
 size_t tile_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
-hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream);
+hipError_t launch_tile(const MoeParams &p, int stages, void *workspace, hipStream_t stream);
 
 // Wide kernel for large batches: macro blocks of up to 256 consecutive sorted rows of one expert (several row blocks),
 // twice the tokens per weight byte of the tile kernel; same per-slot result rows and reduce kernel.  block_m > 32.
 bool wide_supported(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
 size_t wide_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m);
-hipError_t launch_wide(const MoeParams &p, void *workspace, hipStream_t stream);
+hipError_t launch_wide(const MoeParams &p, int stages, void *workspace, hipStream_t stream);
 
 // out[t] = bf16(out[t] + sum over the token's live slots of y[slot]) (or bf16(sum) when p.overwrite); closes the
 // workspace's launch epoch.  Shared by the tile and wide kernels, which write each (token, slot) row once into y.

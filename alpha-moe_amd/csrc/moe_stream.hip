@@ -98,32 +98,6 @@ __device__ __forceinline__ Routing<TM> load_routing(const MoeParams &p, int mb, 
     return r;
 }
 
-// Measurement builds only (-DALPHA_MOE_STREAM_TRACE, microbench/stream_item_timeline.py): every item leaves four words
-// - kind, workgroup and index; start; end of its wait (DOWN, FIN) or of its streaming (UP); end - of the 100 MHz
-// clock in a device array that alpha_moe_debug_trace_read() hands to the host.  The library is built without the macro.
-#ifdef ALPHA_MOE_STREAM_TRACE
-__device__ unsigned long long g_trace[1 << 16][4];
-__device__ int g_trace_n;
-#define TRACE_VARS unsigned long long tr_t0 = 0, tr_t1 = 0
-#define TRACE_BEGIN tr_t0 = tr_t1 = wall_clock64()
-#define TRACE_MARK tr_t1 = wall_clock64()
-#define TRACE_END(kind, idx)                                                                                          \
-    if (threadIdx.x == 0) {                                                                                           \
-        const int slot_ = atomicAdd(&g_trace_n, 1);                                                                   \
-        if (slot_ < (1 << 16)) {                                                                                      \
-            g_trace[slot_][0] = ((unsigned long long)(kind) << 56) | ((unsigned long long)blockIdx.x << 32) | (unsigned)(idx); \
-            g_trace[slot_][1] = tr_t0;                                                                                \
-            g_trace[slot_][2] = tr_t1;                                                                                \
-            g_trace[slot_][3] = wall_clock64();                                                                       \
-        }                                                                                                             \
-    }
-#else
-#define TRACE_VARS
-#define TRACE_BEGIN
-#define TRACE_MARK
-#define TRACE_END(kind, idx)
-#endif
-
 // TM: 16-token tiles per row block; WN: wavefronts per workgroup; S: 2 KiB tiles in each wavefront's LDS ring
 template <int TM, int WN, int S>
 __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
@@ -150,7 +124,6 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     __shared__ float s_amax[WN][TM * 16];
     __shared__ int s_bcast[2];
 
-    TRACE_VARS;
     const MoeParams &p = s.p;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -360,7 +333,6 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         }
         fetch_next();
         drain_vmem();
-        TRACE_MARK;
 
         if (s.ks > 1) {
             // K-split: store the valid tokens' partial sums to this item's slice; the last arrival adds the slices up
@@ -519,7 +491,6 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             // everything issued so far (the ring's first S-1 tiles, the activation tiles) has landed
             drain_vmem();
             __syncthreads();
-            TRACE_MARK;
 
             // Result rows are kept in registers and stored NG column groups at a time, normally once, behind the
             // item's last tile: the wait counter that tells a wavefront that a ring tile has landed counts stores as
@@ -572,7 +543,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
     };
 
     // FIN item: two dependent round trips.  (1) Wavefront 0 polls the DOWN counter; an expired wait anywhere in this
-    // launch has added kExpiredBit to that very counter, and lane 1 reads the sticky error word of earlier launches
+    // launch has set kExpiredBit in that very counter, and lane 1 reads the sticky error word of earlier launches
     // with the same instruction.  (2) The stamps of the token's slots, the rows of ALL its slots and the prior output
     // go out together; rows of slots that are not live this launch are dropped after the fact (they are stale bytes of
     // this workspace, nothing else).
@@ -591,11 +562,10 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             if (lane == 0) {
                 if (!up) store_agent(&s.ctl->error, 1);
                 // a result row may be missing: the output says so itself, NaN in every element
-                s_bcast[1] = !up || __builtin_amdgcn_readlane(v, 1) != 0 || (__builtin_amdgcn_readlane(v, 0) >> 30) != 0;
+                s_bcast[1] = !up || __builtin_amdgcn_readlane(v, 1) != 0 || (__builtin_amdgcn_readlane(v, 0) & kExpiredBit) != 0;
             }
         }
         __syncthreads();
-        TRACE_MARK;
         // an item sums fin_w (1 or 2) chunks of 1024 columns: with more chunks than workgroups, two per item halve the
         // rounds of dependent memory round trips that close the call
         const bool poisoned = s_bcast[1] != 0;
@@ -703,13 +673,11 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
         __syncthreads();
     }
     while (item < total) {
-        TRACE_BEGIN;
         next_item = -1;
         const int kind = run_item(item);
         (void)kind;
         fetch_next();   // paths that did not get there themselves (skipped blocks, FIN items)
         __syncthreads();
-        TRACE_END(kind, item);
         if (tid == 0) s_bcast[0] = next_item;
         __syncthreads();
         item = __builtin_amdgcn_readfirstlane(s_bcast[0]);
@@ -906,21 +874,6 @@ hipError_t resident_slots(const Variant &v, int lds_bytes, int *slots)
 }
 
 }  // namespace
-
-#ifdef ALPHA_MOE_STREAM_TRACE
-extern "C" int alpha_moe_debug_trace_read(void *dst, int max_records)
-{
-    int n = 0;
-    (void)hipDeviceSynchronize();
-    (void)hipMemcpyFromSymbol(&n, HIP_SYMBOL(g_trace_n), sizeof(int));
-    if (n > max_records) n = max_records;
-    if (n > (1 << 16)) n = 1 << 16;
-    (void)hipMemcpyFromSymbol(dst, HIP_SYMBOL(g_trace), (size_t)n * 32);
-    const int zero = 0;
-    (void)hipMemcpyToSymbol(HIP_SYMBOL(g_trace_n), &zero, sizeof(int));
-    return n;
-}
-#endif
 
 size_t stream_prefix_bytes() { return align_up(kPrefixBytes); }
 

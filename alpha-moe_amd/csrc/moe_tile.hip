@@ -48,24 +48,6 @@ constexpr int kStages = 3;
 constexpr int kARingBytes = 4 * kStages * 8192;   // 4 wavefronts x 3 stages x 4 tiles of 2 KiB
 constexpr int kMaxTailBytes = 48 << 10;           // token-tile ring / requantised tiles next to the weight rings
 
-// Measurement builds only (-DALPHA_MOE_TILE_PROBE=<bits>, microbench/tile_phase_probe.py): parts of the kernel are
-// compiled out to time the rest.  Results are then wrong on purpose.  The library is built without the macro, and
-// every TILE_PROBE() below is then a constant false.
-enum : int {
-    kProbeNoUp = 1,       // up/gate items only stamp their flag
-    kProbeNoDown = 2,     // down items are skipped
-    kProbeNoY = 4,        // down items do not store their result rows
-    kProbeNoReduce = 8,   // the reduce kernel is not launched
-    kProbeRow0 = 16,      // every routed row gathers token 0 (token tiles come from L2)
-    kProbeExpert8 = 32,   // expert e reads the weights of expert e % 8 (weights come from L2 / Infinity Cache)
-    kProbeNoLoad = 64,    // up/gate items issue no loads (matrix work on whatever LDS holds)
-    kProbeNoMma = 128,    // steps issue their loads and do no matrix or vector work
-};
-#ifndef ALPHA_MOE_TILE_PROBE
-#define ALPHA_MOE_TILE_PROBE 0
-#endif
-#define TILE_PROBE(bits) (((ALPHA_MOE_TILE_PROBE) & (bits)) != 0)
-
 struct TileParams {
     MoeParams p;
     StreamCtl *ctl;
@@ -88,15 +70,9 @@ struct TileParams {
 // load instruction blocks its wavefront for 30-60 ns (measured), and the other wavefront of the SIMD computes then.
 template <int TH, int NOPS, typename Issue>
 __device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *b_tiles, const float *row, float sc0,
-                                         float sc1, v4f (&acc)[4][TH], int frag_lo, int frag_hi, Issue issue,
-                                         bool loads_only = false)
+                                         float sc1, v4f (&acc)[4][TH], int frag_lo, int frag_hi, Issue issue)
 {
     constexpr int GROUPS = 4 * TH;
-    if (loads_only) {   // constant false outside measurement builds
-#pragma unroll
-        for (int i = 0; i < NOPS; i++) issue(i);
-        return;
-    }
     auto read_tile = [&](const uint8_t *tile) -> v8i {
         return cat(*reinterpret_cast<const v4i *>(tile + frag_lo), *reinterpret_cast<const v4i *>(tile + frag_hi));
     };
@@ -211,14 +187,13 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
     auto up_item = [&](int mb, int ib) {
         int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
         if (e < 0 || e >= p.E) return;
-        if (TILE_PROBE(kProbeExpert8)) e &= 7;
         const bool nt = lone_block(mb, e);
         if (tid < TM * 16) {
             const int idx = mb * p.block_m + tid;
             int id = -1;
             if (tid < p.block_m && idx < p.sorted_num) id = p.sorted_ids[idx];
             const int tk = id / p.top_k;
-            s_tok[tid] = (id >= 0 && tk < p.M && !TILE_PROBE(kProbeRow0)) ? tk : 0;
+            s_tok[tid] = (id >= 0 && tk < p.M) ? tk : 0;
         }
         // this slice's gate (row 2*ib) and up (row 2*ib+1) scale rows
         {
@@ -241,7 +216,6 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         // operation i of a step's OPS1: weight tile half (i < AOPS), token tile half, token scales
         auto issue_op = [&](int kb, int stage, int i) {
             const int kc = kb < nkb ? kb : nkb - 1;
-            if (TILE_PROBE(kProbeNoLoad)) return;
             if (i < AOPS) {
                 const int up = i >> 1, h = i & 1;
                 const uint8_t *src = wbase + (h * 16 + 8 * up) * p.w_rs + kc * p.w_ks + ld_chunk[h];
@@ -280,8 +254,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
                     lds_barrier();
                     mma_step<TH, OPS1>(a_ring + h * 8192, xbuf + h * (TM * 2048) + g * (TH * 2048),
                                        &s_xs[h][g * (TH * 16) + n], s_ws[0][kb], s_ws[1][kb], acc, frag_lo, frag_hi,
-                                       [&](int i) { issue_op(kb + 2, (h + 2) % kStages, i); },
-                                       TILE_PROBE(kProbeNoMma));
+                                       [&](int i) { issue_op(kb + 2, (h + 2) % kStages, i); });
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -434,14 +407,14 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
                     const float ws2 = s_w2s[(c0 >> 7) * n_ib + cib];
                     mma_step<THD, AOPS>(a_ring + h * 8192, aq + cib * (TMD * 2048) + g * (THD * 2048),
                                         &s_sa[cib][g * (THD * 16) + n], ws2, ws2, accd, frag_lo, frag_hi,
-                                        [&](int i) { issue2_op((h + 2) % kStages, i); }, TILE_PROBE(kProbeNoMma));
+                                        [&](int i) { issue2_op((h + 2) % kStages, i); });
                     advance2();
                     __builtin_amdgcn_sched_barrier(0);
                     cib++;
                     if (cib == n_ib) {
 #pragma unroll
                         for (int t = 0; t < THD; t++) {
-                            if (valid[t] && cg < my_groups && !TILE_PROBE(kProbeNoY)) {
+                            if (valid[t] && cg < my_groups) {
                                 uint16_t *yp = s.y + (size_t)slot[t] * K + c0 + 16 * q;
 #pragma unroll
                                 for (int half = 0; half < 2; half++) {
@@ -532,12 +505,8 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
             down = (nb - lag) * per_down + (item - head_items - mid_items);
         }
         if (up >= 0) {
-            if (!TILE_PROBE(kProbeNoUp)) {
-                up_item(qi * per_q + up / per_up, up % per_up);
-            } else if (tid == 0) {
-                store_agent(&s.flag[(qi * per_q + up / per_up) * n_ib + up % per_up], epoch);
-            }
-        } else if (!TILE_PROBE(kProbeNoDown)) {
+            up_item(qi * per_q + up / per_up, up % per_up);
+        } else {
             run_down(qi * per_q + down / per_down, down % per_down);
         }
         __syncthreads();   // everybody is done with the item's LDS tables and rings before the next item refills them
@@ -659,13 +628,14 @@ hipError_t allow_dynamic_lds(int th, TileFn fn)
 
 }  // namespace
 
-// 64-column groups per DOWN item: about 14 ring steps (a step is one group x one slice), a multiple of 4 so that
-// every pair of wavefronts gets the same number of groups
-static int groups_per_item(int n_ib)
+// 64-column groups per DOWN item: about 5 * stages ring steps (a step is one group x one slice; 14 at stages = 3), a
+// multiple of 4 so that every pair of wavefronts gets the same number of groups
+static int groups_per_item(int n_ib, int stages)
 {
     const int e = tunable(kTunTileGps, 0);
     if (e > 0) return (e + 3) / 4 * 4;
-    return 4 * ((14 + n_ib - 1) / n_ib);
+    const int steps = stages == 3 ? 14 : 5 * stages;
+    return 4 * ((steps + n_ib - 1) / n_ib);
 }
 
 bool tile_supported(int top_k, int M, int K, int N, int E, int sorted_num, int block_m)
@@ -687,7 +657,7 @@ size_t tile_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_nu
            align_up(n_mb * (N / 256) * tm * 2048) + align_up(n_mb * (N / 256) * tm * 16 * sizeof(float));
 }
 
-hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
+hipError_t launch_tile(const MoeParams &p, int stages, void *workspace, hipStream_t stream)
 {
     uint8_t *ws = static_cast<uint8_t *>(workspace);
     TileParams s;
@@ -705,7 +675,7 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
     s.aqs = ws + off;
     off += align_up((size_t)s.n_mb_max * s.n_ib * tm * 2048);
     s.sas = reinterpret_cast<float *>(ws + off);
-    s.gps = groups_per_item(s.n_ib);
+    s.gps = groups_per_item(s.n_ib, stages);
     s.n_cs = ((p.K >> 6) + s.gps - 1) / s.gps;
     // up/gate items of this many row blocks run ahead of the first down items of a queue: with ~32 workgroups
     // on a queue, a down item's up/gate items were taken at least two rounds of the queue earlier
@@ -732,7 +702,6 @@ hipError_t launch_tile(const MoeParams &p, void *workspace, hipStream_t stream)
     hipLaunchKernelGGL(fn, dim3((unsigned)grid), dim3(512), lds_bytes, stream, s);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
-    if (TILE_PROBE(kProbeNoReduce)) return hipSuccess;
     RowsReduce r;
     r.p = p;
     r.ctl = s.ctl;

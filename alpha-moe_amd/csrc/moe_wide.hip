@@ -61,10 +61,6 @@ struct WideParams {
     int w_nt;               // weights with non-temporal loads: 1 always, 0 never, -1 for experts with one macro block
 };
 
-#ifndef WIDE_PROBE   // PROBE
-#define WIDE_PROBE 0   // PROBE
-#endif   // PROBE
-#define WPROBE(b) (((WIDE_PROBE) & (b)) != 0)   // PROBE: 1 no up, 2 no down, 4 no y, 8 no reduce, 64 no loads, 128 no mma
 __device__ __forceinline__ int rfl(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // A wavefront-uniform pointer the compiler cannot fold into per-lane address arithmetic: added to a 32-bit per-lane
@@ -173,7 +169,7 @@ __device__ __forceinline__ void wide_step(const uint8_t *a_tiles, const uint8_t 
             // per-token factors of tile tt sit at (tt & 7) * 32 + (tt >> 3) * 16; tt = 2 t + g, g folded into `row`
             f_next = row[(t + 1) < 4 ? (t + 1) * 64 : (t + 1 - 4) * 64 + 16];
         }
-        if (t < nt_w && !WPROBE(128)) {
+        if (t < nt_w) {
             const float p0 = f * sc0, p1 = f * sc1;
             v4f prev;
 #pragma unroll
@@ -192,6 +188,74 @@ __device__ __forceinline__ void wide_step(const uint8_t *a_tiles, const uint8_t 
         }
         b = b_next;
         f = f_next;
+    }
+}
+
+// Half a step: token tiles T0 .. T0 + 3 of the wavefront against weight fragments already in registers.  Same
+// arithmetic and order as wide_step.
+template <int T0, typename Issue>
+__device__ __forceinline__ void wide_half(const v8i (&a)[4], const uint8_t *b_tiles, const float *row, float sc0,
+                                          float sc1, v4f (&acc)[4][8], int frag_lo, int frag_hi, int nt_w, Issue issue)
+{
+    auto read_tile = [&](const uint8_t *tile) -> v8i {
+        return cat(*reinterpret_cast<const v4i *>(tile + frag_lo), *reinterpret_cast<const v4i *>(tile + frag_hi));
+    };
+    auto row_at = [&](int t) { return row[t < 4 ? t * 64 : (t - 4) * 64 + 16]; };
+    v8i b = read_tile(b_tiles + T0 * 4096);
+    float f = row_at(T0);
+#pragma unroll
+    for (int t = T0; t < T0 + 4; t++) {
+        issue(t);
+        v8i b_next = b;
+        float f_next = f;
+        if (t + 1 < T0 + 4) {
+            b_next = read_tile(b_tiles + (t + 1) * 4096);
+            f_next = row_at(t + 1);
+        }
+        if (t < nt_w) {
+            const float p0 = f * sc0, p1 = f * sc1;
+            v4f prev;
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const v4f cur = mfma_fp8(a[k], b);
+                __builtin_amdgcn_sched_barrier(0);
+                if (k > 0) {
+                    acc[k - 1][t] += prev * (((k - 1) & 1) ? p1 : p0);
+                    asm volatile("" : "+v"(acc[k - 1][t]));
+                }
+                prev = cur;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            acc[3][t] += prev * p1;
+            asm volatile("" : "+v"(acc[3][t]));
+        }
+        b = b_next;
+        f = f_next;
+    }
+}
+
+// "At most n of this wavefront's loads are still outstanding", n known only at run time (the same for all lanes).
+// Loads complete in the order they were issued, so this is "every load issued before the last n has landed".
+__device__ __forceinline__ void wait_pending(int n)
+{
+    switch (n) {
+    case 0: wait_vmcnt<0>(); break;
+    case 1: wait_vmcnt<1>(); break;
+    case 2: wait_vmcnt<2>(); break;
+    case 3: wait_vmcnt<3>(); break;
+    case 4: wait_vmcnt<4>(); break;
+    case 5: wait_vmcnt<5>(); break;
+    case 6: wait_vmcnt<6>(); break;
+    case 7: wait_vmcnt<7>(); break;
+    case 8: wait_vmcnt<8>(); break;
+    case 9: wait_vmcnt<9>(); break;
+    case 10: wait_vmcnt<10>(); break;
+    case 11: wait_vmcnt<11>(); break;
+    case 12: wait_vmcnt<12>(); break;
+    case 13: wait_vmcnt<13>(); break;
+    case 14: wait_vmcnt<14>(); break;
+    case 15: wait_vmcnt<15>(); break;
+    default: wait_vmcnt<16>(); break;
     }
 }
 
@@ -276,7 +340,7 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
             const int tk = id / p.top_k;
             const bool ok = id >= 0 && tk < p.M;
             if (!for_down) {
-                s_tok[tid] = ok ? (WPROBE(16) ? 0 : tk) : -1;
+                s_tok[tid] = ok ? tk : -1;
             } else {
                 s_tok[tid] = ok ? id : -1;
                 s_tw[tid] = ok ? p.topk_w[id] * p.scaling : 0.f;
@@ -308,7 +372,7 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
         const int unit = mc.mb0 * n_ib + ib;
         if (n_tiles > 0) {
             // token-tile gather: wavefront v loads tiles v and v + 8
-            unsigned x_off[2][2], xs_off;
+            unsigned x_off[2][2], xs_off[2];
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
@@ -316,9 +380,10 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
                     const int tk = s_tok[(wave + 8 * j) * 16 + 8 * h + ld_row];
                     x_off[j][h] = (unsigned)(tk < 0 ? 0 : tk) * (unsigned)K + ld_chunk[h];
                 }
-            {
-                const int tk = s_tok[(wave + 8 * ((lane >> 4) & 1)) * 16 + n];
-                xs_off = (unsigned)(tk < 0 ? 0 : tk) * (unsigned)nkb;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int tk = s_tok[(wave + 8 * j) * 16 + n];
+                xs_off[j] = (unsigned)(tk < 0 ? 0 : tk) * (unsigned)nkb;
             }
             // Weight rows of the pair: tile a = (32-row group a / 2, gate | up a % 2); matrix row r of the tile is slab
             // row group * 32 + (r / 8) * 16 + r % 8 (+ 8 for up), so load h of a tile covers slab rows ... + 16 h +
@@ -330,70 +395,87 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
                 for (int h = 0; h < 2; h++)
                     w_off[up][h] =
                         (unsigned)((ib * 256 + w * 64 + g * 32 + ld_row + h * 16 + 8 * up) * p.w_rs) + ld_chunk[h];
-            const uint8_t *wexp = p.w + (size_t)(WPROBE(32) ? mc.e & 7 : mc.e) * p.N * K;
+            const uint8_t *wexp = p.w + (size_t)mc.e * p.N * K;
             const bool nt = mc.lone;
-            // operation i of a step: 4 weight tile halves, 4 token tile halves, the token scales
-            auto issue_op = [&](int kb, int stage, int i) {
-                if (WPROBE(64)) return;   // PROBE
-                if (i < 4) {
-                    const int up = i >> 1, h = i & 1;
-                    const uint8_t *src = wexp + (size_t)kb * p.w_ks;
-                    uint8_t *dst = a_ring + stage * kWStageA + w * 8192 + (2 * g + up) * 2048 + h * 1024;
-                    if (nt) dma16_sv<2>(src, w_off[up][h], dst);
-                    else dma16_sv<0>(src, w_off[up][h], dst);
-                } else if (i < 8) {
-                    const int j = (i - 4) >> 1, h = i & 1;
-                    if (wave + 8 * j < n_tiles)
-                        dma16_sv<0>(p.x + (size_t)kb * 128, x_off[j][h],
-                                    xbuf + stage * kWStageX + (wave + 8 * j) * 2048 + h * 1024);
-                } else {
-                    if (lane < 32) dma4_sv<0>(p.x_scale + kb, xs_off * 4u, &s_xs[stage][wave * 32]);
+            // Loads of a step, in three groups that are issued - and waited for - separately:
+            //   A    the wavefront's 4 weight tile halves
+            //   XLO  token tile `wave` (tiles 0..7: the first half of a step) and its scales
+            //   XHI  token tile `wave + 8` and its scales
+            // `issued` counts this wavefront's load instructions; a group's mark is the count right after its last one.
+            int issued = 0;
+            auto issue_a_op = [&](int kb, int stage, int i) {   // i < 4
+                const int up = i >> 1, h = i & 1;
+                const uint8_t *src = wexp + (size_t)kb * p.w_ks;
+                uint8_t *dst = a_ring + stage * kWStageA + w * 8192 + (2 * g + up) * 2048 + h * 1024;
+                if (nt) dma16_sv<2>(src, w_off[up][h], dst);
+                else dma16_sv<0>(src, w_off[up][h], dst);
+                issued++;
+            };
+            auto issue_x_op = [&](int kb, int stage, int j, int i) {   // i < 3: two tile halves, the scales
+                if (wave + 8 * j >= n_tiles) return;
+                if (i < 2) {
+                    dma16_sv<0>(p.x + (size_t)kb * 128, x_off[j][i],
+                                xbuf + stage * kWStageX + (wave + 8 * j) * 2048 + i * 1024);
+                } else if (lane < 16) {
+                    dma4_sv<0>(p.x_scale + kb, xs_off[j] * 4u, &s_xs[stage][wave * 32 + 16 * j]);
                 }
+                issued++;
             };
             clear_acc();
-#if (WIDE_PROBE & 0x300)   // PROBE: loads only, 2 or 3 steps in flight (LDS contents are garbage)
-            {   // PROBE
-                constexpr int D = (WIDE_PROBE & 0x200) ? 3 : 2;   // PROBE
-                for (int d = 0; d < D; d++)   // PROBE
-                    for (int i = 0; i < 9; i++) issue_op(d < nkb ? d : nkb - 1, d & 1, i);   // PROBE
-                for (int kb = 0; kb < nkb; kb++) {   // PROBE
-                    wait_vmcnt<9 * (D - 1)>();   // PROBE
-                    lds_barrier();   // PROBE
-                    for (int i = 0; i < 9; i++) issue_op(kb + D < nkb ? kb + D : nkb - 1, kb & 1, i);   // PROBE
-                }   // PROBE
-                wait_vmcnt<0>();   // PROBE
-            }   // PROBE
-            if (false)   // PROBE
-#endif   // PROBE
-            {
-#pragma unroll
-            for (int i = 0; i < 9; i++) issue_op(0, 0, i);
-            wait_vmcnt<0>();
+            // Step kb reads stage kb & 1.  Its weight tiles are in registers right after the step's first barrier, so the
+            // weight stage is refilled (step kb + 2) behind a second barrier; the first half of the token stage is
+            // refilled behind a third one in the middle of the step, the second half from the start of the next step.
+            // The loads go out one at a time between the matrix instructions of the token tiles: a load instruction
+            // holds its wavefront until the memory pipeline takes it, and a burst of them holds the matrix work up.
+            int mark_a[2], mark_lo[2], mark_hi[2];
+            for (int i = 0; i < 4; i++) issue_a_op(0, 0, i);
+            mark_a[0] = issued;
+            for (int i = 0; i < 3; i++) issue_x_op(0, 0, 0, i);
+            mark_lo[0] = issued;
+            for (int i = 0; i < 3; i++) issue_x_op(0, 0, 1, i);
+            mark_hi[0] = issued;
+            if (nkb > 1) {
+                for (int i = 0; i < 4; i++) issue_a_op(1, 1, i);
+                mark_a[1] = issued;
+                for (int i = 0; i < 3; i++) issue_x_op(1, 1, 0, i);
+                mark_lo[1] = issued;
             }
-            for (int kb0 = 0; kb0 < nkb && !(WIDE_PROBE & 0x300); kb0 += 2) {
+            for (int kb0 = 0; kb0 < nkb; kb0 += 2) {
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
                     const int kb = kb0 + h;
                     if (kb < nkb) {
-                        lds_barrier();
-                        wide_step(a_ring + h * kWStageA + w * 8192, xbuf + h * kWStageX + g * 2048, &s_xs[h][row_off],
-                                  s_ws[0][kb], s_ws[1][kb], acc, frag_lo, frag_hi, nt_w, [&](int t) {
-                                      if (kb + 1 < nkb) {
-                                          // 9 loads over the first four token tiles: 3, 2, 2, 2
-                                          if (t == 0) {
-                                              issue_op(kb + 1, h ^ 1, 0);
-                                              issue_op(kb + 1, h ^ 1, 4);
-                                              issue_op(kb + 1, h ^ 1, 8);
-                                          } else if (t < 4) {
-                                              issue_op(kb + 1, h ^ 1, t);
-                                              issue_op(kb + 1, h ^ 1, t + 4);
-                                          }
-                                      }
-                                  });
-                        wait_vmcnt<0>();
+                        wait_pending(issued - mark_a[h]);
+                        lds_barrier();   // everybody's weight tiles of step kb have landed; step kb - 1 is done with
+                        v8i a[4];
+                        {
+                            const uint8_t *a_tiles = a_ring + h * kWStageA + w * 8192;
+#pragma unroll
+                            for (int k = 0; k < 4; k++)
+                                a[k] = cat(*reinterpret_cast<const v4i *>(a_tiles + k * 2048 + frag_lo),
+                                           *reinterpret_cast<const v4i *>(a_tiles + k * 2048 + frag_hi));
+                        }
+                        wait_pending(issued - mark_lo[h]);
+                        lds_barrier();   // weight fragments are in registers everywhere; token tiles 0..7 have landed
+                        const float sc0 = s_ws[0][kb], sc1 = s_ws[1][kb];
+                        wide_half<0>(a, xbuf + h * kWStageX + g * 2048, &s_xs[h][row_off], sc0, sc1, acc, frag_lo,
+                                     frag_hi, nt_w, [&](int t) {
+                                         if (kb + 2 < nkb) issue_a_op(kb + 2, h, t);
+                                         if (kb + 1 < nkb && t < 3) issue_x_op(kb + 1, h ^ 1, 1, t);
+                                     });
+                        mark_a[h] = issued;        // (a load of step kb + 1's second half may follow the last weight
+                        mark_hi[h ^ 1] = issued;   //  load: waiting for one more than needed is harmless)
+                        wait_pending(issued - mark_hi[h]);
+                        lds_barrier();   // everybody is done with token tiles 0..7; tiles 8..15 have landed
+                        wide_half<4>(a, xbuf + h * kWStageX + g * 2048, &s_xs[h][row_off], sc0, sc1, acc, frag_lo,
+                                     frag_hi, nt_w, [&](int t) {
+                                         if (kb + 2 < nkb && t < 7) issue_x_op(kb + 2, h, 0, t - 4);
+                                     });
+                        mark_lo[h] = issued;
                     }
                 }
             }
+            wait_vmcnt<0>();
 
             // SwiGLU, per-token amax over the slice's 128 columns, FP8 requant into operand tiles
 #pragma unroll
@@ -479,7 +561,6 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
         // operation i of the step (lg, lib) into ring stage `stage`: 4 w2 tile halves; streamed: 4 requantised tile
         // halves of slice lib and their scales
         auto issue_op = [&](int stage, int i) {
-            if (WPROBE(64)) return;   // PROBE
             if (i < 4) {
                 const int kk = i >> 1, h = i & 1;
                 const int c0 = group_of(lg) << 6;
@@ -577,7 +658,7 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
                             if (t < nt_w) {
                                 const int r = (2 * t + g) * 16 + n;
                                 const int slot = s_tok[r];
-                                if (slot >= 0 && cg < my_groups && !WPROBE(4)) {
+                                if (slot >= 0 && cg < my_groups) {
                                     const float tw = s_tw[r];
                                     uint16_t *yp = s.y + (size_t)slot * K + c0 + 16 * q;
 #pragma unroll
@@ -655,9 +736,7 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
             down = (nb - lag) * per_down + (item - head_items - mid_items);
         }
         if (up >= 0) {
-            if (!WPROBE(1)) up_item(qi * per_q + up / per_up, up % per_up);
-            else if (tid == 0) store_agent(&s.flag[rfl(s.plan[1 + qi * per_q + up / per_up]) * n_ib + up % per_up], epoch);   // PROBE
-        } else if (WPROBE(2)) {   // PROBE
+            up_item(qi * per_q + up / per_up, up % per_up);
         } else if (n_ib <= kWResidentIb) {
             down_item(qi * per_q + down / per_down, down % per_down, std::true_type());
         } else {
@@ -691,13 +770,13 @@ hipError_t allow_dynamic_lds()
     return err;
 }
 
-// 64-column groups per DOWN item: about 16 ring steps (a step is four groups x one slice), a multiple of 4 so that
-// every pair of wavefronts gets the same number of groups
-int groups_per_item(int n_ib)
+// 64-column groups per DOWN item: about 8 * stages ring steps (a step is four groups x one slice), a multiple of 4 so
+// that every pair of wavefronts gets the same number of groups
+int groups_per_item(int n_ib, int stages)
 {
     const int e = tunable(kTunTileGps, 0);
     if (e > 0) return (e + 3) / 4 * 4;
-    return 4 * ((16 + n_ib - 1) / n_ib);
+    return 4 * ((8 * stages + n_ib - 1) / n_ib);
 }
 
 }  // namespace
@@ -721,7 +800,7 @@ size_t wide_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_nu
            align_up((n_mb + 1) * sizeof(int));
 }
 
-hipError_t launch_wide(const MoeParams &p, void *workspace, hipStream_t stream)
+hipError_t launch_wide(const MoeParams &p, int stages, void *workspace, hipStream_t stream)
 {
     uint8_t *ws = static_cast<uint8_t *>(workspace);
     WideParams s;
@@ -743,7 +822,7 @@ hipError_t launch_wide(const MoeParams &p, void *workspace, hipStream_t stream)
     s.sas = reinterpret_cast<float *>(ws + off);
     off += align_up((size_t)s.n_ib * s.n_tiles_total * 16 * sizeof(float));
     s.plan = reinterpret_cast<int *>(ws + off);
-    s.gps = groups_per_item(s.n_ib);
+    s.gps = groups_per_item(s.n_ib, stages);
     s.n_cs = ((p.K >> 6) + s.gps - 1) / s.gps;
     s.lag = tunable(kTunTileLag, 32);
     s.w_nt = tunable(kTunTileNt, -1);
@@ -767,7 +846,6 @@ hipError_t launch_wide(const MoeParams &p, void *workspace, hipStream_t stream)
     hipLaunchKernelGGL(moe_wide_kernel, dim3((unsigned)grid), dim3(512), kWDynLds, stream, s);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
-    if (WPROBE(8)) return hipSuccess;   // PROBE
     RowsReduce r;
     r.p = p;
     r.ctl = s.ctl;

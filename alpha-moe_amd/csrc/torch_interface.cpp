@@ -26,38 +26,65 @@
 namespace {
 
 // Scratch for the C ABI, one buffer per (device, stream): zero-filled when created and maintained by the library
-// afterwards, so the steady state allocates and clears nothing.  A buffer is never freed or shrunk once a call has
-// used it: a HIP graph captured earlier may hold its address, and its replays keep writing the control block, flags
-// and result rows there.  When a later call needs more, a new buffer of exactly that size takes over for eager calls
-// and the old one stays alive beside it (graphs captured before keep replaying into it).  Growth while the stream is
-// being captured is refused: the fill of the new buffer's control prefix would be recorded into the graph and run on
-// every replay, and the allocation would belong to the graph's private pool.  reserve_workspace() sizes the buffer
-// ahead of time.
+// afterwards, so the steady state allocates and clears nothing.  When a call needs more than the buffer holds, a new one
+// of at least 1.5 times the old size takes over (geometric growth: a stream that sees growing sizes reallocates a
+// logarithmic number of times).  What happens to the old one depends on whether a HIP graph may hold its address: a
+// buffer that was handed out while its stream was being captured is kept alive beside the new one (graphs captured
+// before keep replaying into it: control block, flags and result rows); a buffer only eager calls ever used is dropped,
+// which is safe because the caching allocator hands its memory out again in stream order, behind the kernels that used it.
+// Growth while the stream is being captured is refused: the fill of the new buffer's control prefix would be recorded
+// into the graph and run on every replay, and the allocation would belong to the graph's private pool.
+// reserve_workspace() sizes the buffer ahead of time.
 struct StreamScratch {
     at::Tensor current;
+    bool current_seen_by_capture = false;
     std::vector<at::Tensor> retired;
 };
 
+std::mutex g_scratch_mu;
+std::map<std::pair<int, void *>, StreamScratch> g_scratch;
+
 at::Tensor workspace_for(const at::Device &dev, hipStream_t stream, size_t bytes)
 {
-    static std::mutex mu;
-    static std::map<std::pair<int, void *>, StreamScratch> cache;
-    std::lock_guard<std::mutex> lock(mu);
-    StreamScratch &slot = cache[{dev.index(), static_cast<void *>(stream)}];
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    StreamScratch &slot = g_scratch[{dev.index(), static_cast<void *>(stream)}];
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    (void)hipStreamIsCapturing(stream, &capturing);
     if (!slot.current.defined() || static_cast<size_t>(slot.current.numel()) < bytes) {
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        (void)hipStreamIsCapturing(stream, &capturing);
         TORCH_CHECK(capturing == hipStreamCaptureStatusNone,
                     "alpha_moe: this call needs ", bytes, " bytes of scratch memory on a stream that is being captured "
                     "and holds ", slot.current.defined() ? slot.current.numel() : 0, ": run the operator once with "
                     "these sizes before the capture, or call torch.ops.alpha_moe.reserve_workspace(x, bytes) there");
-        if (slot.current.defined()) slot.retired.push_back(slot.current);
-        const size_t cap = (bytes + 255) & ~static_cast<size_t>(255);
+        size_t cap = bytes;
+        if (slot.current.defined()) {
+            cap = std::max(cap, static_cast<size_t>(slot.current.numel()) * 3 / 2);
+            if (slot.current_seen_by_capture) slot.retired.push_back(slot.current);
+        }
+        cap = (cap + 255) & ~static_cast<size_t>(255);
+        slot.current = at::Tensor();   // an eager-only buffer goes back to the allocator before the new one is taken
         slot.current = at::empty({static_cast<int64_t>(cap)}, at::TensorOptions().dtype(at::kByte).device(dev));
+        slot.current_seen_by_capture = false;
         // only the control block, counters and flags have to start at zero (1.5 MiB, not the whole buffer)
         slot.current.narrow(0, 0, static_cast<int64_t>(alpha_moe_workspace_zero_bytes())).zero_();
     }
+    if (capturing != hipStreamCaptureStatusNone) slot.current_seen_by_capture = true;
     return slot.current;
+}
+
+// scratch_buffers(like): [buffers alive, bytes of the current one, bytes kept for earlier graph captures] of
+// (like's device, the current stream) - for tests and memory accounting.
+std::vector<int64_t> scratch_buffers(const at::Tensor &like)
+{
+    TORCH_CHECK(like.is_cuda(), "scratch_buffers: `like` must be a GPU tensor (it names the device)");
+    const c10::hip::OptionalHIPGuardMasqueradingAsCUDA device_guard(like.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream();
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    auto it = g_scratch.find({like.device().index(), static_cast<void *>(stream)});
+    if (it == g_scratch.end()) return {0, 0, 0};
+    int64_t retired = 0;
+    for (const at::Tensor &t : it->second.retired) retired += t.numel();
+    return {static_cast<int64_t>(it->second.retired.size()) + (it->second.current.defined() ? 1 : 0),
+            it->second.current.defined() ? it->second.current.numel() : 0, retired};
 }
 
 // reserve_workspace(like, bytes): make the scratch buffer of (like's device, the current stream) at least `bytes`
@@ -271,6 +298,8 @@ TORCH_LIBRARY_FRAGMENT(alpha_moe, m)
     m.impl("moe_align_block_size", c10::DispatchKey::CUDA, &moe_align_block_size);
     m.def("reserve_workspace(Tensor like, int bytes) -> ()");
     m.impl("reserve_workspace", c10::DispatchKey::CUDA, &reserve_workspace);
+    m.def("scratch_buffers(Tensor like) -> int[]");
+    m.impl("scratch_buffers", c10::DispatchKey::CUDA, &scratch_buffers);
     m.def("workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_num, int block_m) -> int", &workspace_bytes);
     m.def("fused_moe_w8a8_up_down("
           "Tensor x, Tensor x_scale, Tensor w, Tensor w_scale, Tensor w2, Tensor w2_scale, "

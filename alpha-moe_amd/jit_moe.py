@@ -13,7 +13,10 @@ Differences, all on purpose:
     Infinity Cache (the reference allocates 2 GiB of randn before every call, jit_moe.py:21-22);
   * `--block-ms`, `--stages` and `--num-tests` bound the sweep (the full space is 160 configurations) and `--update`
     merges the result into an existing table;
-  * on MI355X `warp_n` counts 64-wide wavefronts per workgroup and `stages` sizes the LDS ring.
+  * on MI355X the knobs select this: row blocks of at most 32 rows take the streaming kernel (`warp_n` = wavefronts per
+    workgroup, `stages` = depth of each wavefront's LDS ring); above that `warp_n` 4 takes the tile kernel (one row
+    block per item, four token tiles per wavefront), `warp_n` 8 the wide kernel (macro blocks of 256 rows, eight token
+    tiles per wavefront), and `stages` sets the length of their down-projection items.
 """
 import argparse
 import json
@@ -26,9 +29,6 @@ import torch
 HERE = os.path.dirname(os.path.abspath(__file__))
 if HERE not in sys.path:
     sys.path.insert(0, HERE)
-
-import alpha_moe  # noqa: E402,F401  registers torch.ops.alpha_moe.fused_moe_w8a8_up_down
-from alpha_moe_python.prep_hip import moe_align_block_size, per_token_group_quant_fp8  # noqa: E402
 
 _FLUSH = None
 
@@ -60,6 +60,36 @@ def generate_topk_ids(num_experts, num_tokens, top_k, balancedness=1.0):
     return ids.view(num_tokens, top_k)
 
 
+def candidate_list(block_ms, stages):
+    """Every (block_m, block_n, warp_n, stages) of the sweep: the reference's space (jit_moe.py:151-157) restricted to
+    the requested block sizes and stages.  Each combination selects a different kernel variant or item size."""
+    return [(bm, bn, wn, st) for bm in block_ms for (bn, wn) in ((64, 4), (32, 8)) for st in stages]
+
+
+def pick_best(times):
+    """{batch size: {candidate: [mean us per routing sample]}} -> {batch size: table entry}, fastest mean first."""
+    table = {}
+    for nt, val in times.items():
+        timed = [(k, mean(v)) for k, v in val.items() if len(v) > 0]
+        (block_m, bn, wn, stages), best_us = sorted(timed, key=lambda kv: kv[1])[0]
+        print(f"M={nt}: best {(block_m, bn, wn, stages)} {best_us:.1f} us", flush=True)
+        table[nt] = {"block_m": block_m, "block_n": bn, "warp_n": wn, "stages": stages}
+    return table
+
+
+def write_table(path, table, update=False):
+    """The reference's writer (jit_moe.py:181-183): json.dump of {batch size: entry}, so keys come out as strings.
+    update=True keeps the entries `path` already holds for batch sizes not in `table`."""
+    if update and os.path.exists(path):
+        with open(path) as f:
+            merged = {int(k): v for k, v in json.load(f).items()}
+        merged.update(table)
+        table = dict(sorted(merged.items()))
+    with open(path, "w") as f:
+        json.dump(table, f)
+    return table
+
+
 def parse_arguments(argv=None):
     parser = argparse.ArgumentParser(description="MoE autotuner (MI355X)")
     parser.add_argument("--batch-sizes", type=int, nargs="+", default=[8, 32, 128, 256, 512, 1024, 2048, 4096, 8192],
@@ -83,6 +113,8 @@ def parse_arguments(argv=None):
 
 def main(argv=None):
     args = parse_arguments(argv)
+    import alpha_moe  # noqa: F401  registers torch.ops.alpha_moe.fused_moe_w8a8_up_down
+    from alpha_moe_python.prep_hip import moe_align_block_size, per_token_group_quant_fp8
     torch.manual_seed(42)
     dev = "cuda:0"
     top_k = args.top_k + args.shared_expert
@@ -95,9 +127,7 @@ def main(argv=None):
     w1_scale = (torch.randn((E, N // 128, K // 128), dtype=torch.float32) * 0.01).to(dev)
     w2_scale = (torch.randn((E, K // 128, N // 256), dtype=torch.float32) * 0.01).to(dev)
 
-    # row blocks above 32 rows take the tile kernel, which ignores block_n, warp_n and stages: one candidate each
-    candidates = [(bm, bn, wn, st) for bm in args.block_ms if bm <= 32 for (bn, wn) in ((64, 4), (32, 8))
-                  for st in args.stages] + [(bm, 64, 4, 3) for bm in args.block_ms if bm > 32]
+    candidates = candidate_list(args.block_ms, args.stages)
     times = {}
     for num_tokens in args.batch_sizes:
         times[num_tokens] = {c: [] for c in candidates}
@@ -114,6 +144,10 @@ def main(argv=None):
             for block_m, bn, wn, stages in candidates:
                 if num_tokens < block_m and block_m != 16:
                     continue
+                # far from any plausible winner: whole-K streaming items with 8-row blocks at prefill sizes, and
+                # 256-row macro blocks at decode sizes, cost minutes of sweep for nothing
+                if (block_m <= 32 and num_tokens * top_k > 64 * E) or (block_m > 32 and num_tokens * top_k < E):
+                    continue
                 sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(topk_ids, block_m, E)
 
                 def call():
@@ -123,21 +157,8 @@ def main(argv=None):
                 call()
                 times[num_tokens][(block_m, bn, wn, stages)].append(bench_events(call, args.num_tests))
 
-    conf_to_save = {}
-    for nt, val in times.items():
-        timed = [(k, mean(v)) for k, v in val.items() if len(v) > 0]
-        (block_m, bn, wn, stages), best_us = sorted(timed, key=lambda kv: kv[1])[0]
-        print(f"M={nt}: best {(block_m, bn, wn, stages)} {best_us:.1f} us", flush=True)
-        conf_to_save[nt] = {"block_m": block_m, "block_n": bn, "warp_n": wn, "stages": stages}
-
     out_config = args.out_config or f"moe_jit_{E}_{N}_{K}.json"
-    if args.update and os.path.exists(out_config):
-        with open(out_config) as f:
-            merged = {int(k): v for k, v in json.load(f).items()}
-        merged.update(conf_to_save)
-        conf_to_save = dict(sorted(merged.items()))
-    with open(out_config, "w") as f:
-        json.dump(conf_to_save, f)
+    write_table(out_config, pick_best(times), args.update)
     return 0
 
 

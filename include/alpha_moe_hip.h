@@ -122,8 +122,8 @@ int alpha_moe_fused_moe_w8a8_up_down_prepacked(
  * the shipped shard shapes (DeepSeek-V3 shard with the shipped knobs: up to M = 256) but not prefill, whose scratch
  * grows with M * top_k * K.  All calls on one device share the one
  * buffer, which keeps the last call's contents: calls that overlap in time on one device race (order them on one
- * stream), and a bounded wait that ran out stays recorded for the life of the process (every later call then fills
- * `out` with NaN).  The first call on a device looks the buffer's address up; make that call outside graph capture.
+ * stream), and a bounded wait that ran out stays recorded (every later call then fills `out` with NaN) until
+ * alpha_moe_static_scratch_reset clears it.  The first call on a device looks the buffer's address up; make that call outside graph capture.
  */
 #define ALPHA_MOE_STATIC_SCRATCH_BYTES ((size_t)64 << 20)
 int alpha_moe_fused_moe_w8a8_up_down_static(
@@ -136,6 +136,17 @@ int alpha_moe_fused_moe_w8a8_up_down_static(
     int top_k, int M, int K, int N, int num_experts, int sorted_num,
     int block_m, int block_n, int warp_n, int stages,
     float scaling_factor, void *stream /* hipStream_t */);
+
+/*
+ * Health and repair of the built-in scratch buffer of alpha_moe_fused_moe_w8a8_up_down_static on the current device
+ * (callers have no address for it, so alpha_moe_workspace_check cannot be pointed at it).  No counterpart in the
+ * reference.  alpha_moe_static_scratch_check waits for `stream` and returns ALPHA_MOE_ERR_WAIT_EXPIRED if a bounded wait
+ * ever ran out on that buffer, ALPHA_MOE_OK otherwise.  alpha_moe_static_scratch_reset clears the buffer's control
+ * prefix on `stream` (a fill kernel; no allocation), which also clears a recorded expiry: call it with no call on that
+ * device in flight, outside graph capture.
+ */
+int alpha_moe_static_scratch_check(void *stream /* hipStream_t */);
+int alpha_moe_static_scratch_reset(void *stream /* hipStream_t */);
 
 /* Bytes of scratch the calls above need for these sizes (0 if any is not positive). */
 size_t alpha_moe_workspace_bytes(int top_k, int M, int K, int N, int num_experts, int sorted_num, int block_m);
@@ -193,16 +204,6 @@ int alpha_moe_moe_align_block_size(const int32_t *topk_ids, int numel, int num_e
                                    int32_t *sorted_token_ids, int sorted_num, int32_t *expert_ids, int n_blocks,
                                    int32_t *num_tokens_post_padded, void *workspace, size_t workspace_bytes,
                                    void *stream /* hipStream_t */);
-
-/*
- * Tuning overrides, for experiments and tests: `name` is one of ALPHA_MOE_PATH (1 direct, 2 stream, 3 tile),
- * ALPHA_MOE_STRICT_QUEUE, ALPHA_MOE_KBPI, ALPHA_MOE_TPI, ALPHA_MOE_LAG, ALPHA_MOE_GRID,
- * ALPHA_MOE_TILE_GPS, ALPHA_MOE_TILE_LAG, ALPHA_MOE_TILE_GRID, ALPHA_MOE_TILE_NT.  set != 0 installs `value`, set == 0
- * returns the choice to the library.  The environment variables of the same names are read once, when the library is
- * first used; no launch reads the environment.  Not thread-safe against concurrent launches.  Results stay within
- * the parity bar whatever is set.  Returns ALPHA_MOE_ERR_SHAPE for an unknown name.  No counterpart in the reference.
- */
-int alpha_moe_set_tunable(const char *name, int value, int set);
 
 /* Human-readable text for a status code (static storage). */
 const char *alpha_moe_status_string(int status);

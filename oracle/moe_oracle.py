@@ -153,15 +153,39 @@ def _silu_mul(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
     return g / (1.0 + torch.exp(-g)) * u           # K.cu:76-79
 
 
-def _expert_forward(xd, w1_e, w1s_e, w2_e, w2s_e):
+def _up_sums_kblock(xq, xs, w1_e, w1s_e):
+    """The up/gate sums accumulated the way a block-scaled kernel does (K.cu:900-933): per 128-wide K block the
+    exact sum of the FP8 products, rounded to fp32; then h = fma(partial, x_scale * w_scale, h) in fp32, blocks in
+    ascending order.  Same mathematics as one dense fp32 product of the dequantised operands, another rounding order:
+    the two differ in the last bits of h, which matters wherever a value sits on a bf16 rounding boundary."""
+    n, K = xq.shape
+    N = w1_e.shape[0]
+    w = w1_e.float().double()
+    xq = xq.double()
+    h = torch.zeros((n, N), dtype=torch.float32)
+    row_block = torch.arange(N) // 128
+    for kb in range(K // 128):
+        part = (xq[:, kb * 128:(kb + 1) * 128] @ w[:, kb * 128:(kb + 1) * 128].t()).float()     # exact, then one rounding
+        scale = xs[:, kb:kb + 1] * w1s_e[row_block, kb].unsqueeze(0)                             # fp32 product
+        h = (part.double() * scale.double() + h.double()).float()                                # fused multiply-add
+    return h
+
+
+def _expert_forward(xd, w1_e, w1s_e, w2_e, w2s_e, up_sums=None, up_nudge=0.0):
     """fp32 maths of one expert on dequantised activations xd [n, K]; returns y [n, K] before routing weights.
 
-    w1_e / w1s_e are in the ORIGINAL (de-interleaved) row order: gate rows then up rows.
+    w1_e / w1s_e are in the ORIGINAL (de-interleaved) row order: gate rows then up rows.  up_sums: the up/gate sums
+    [n, N] where the caller has accumulated them in another order (_up_sums_kblock).  up_nudge: relative perturbation
+    of those sums before they are rounded to bf16 (see fused_moe_oracle).
     """
     N, K = w1_e.shape
     I = N // 2
-    w1d = w1_e.float() * _expand_block_scale(w1s_e, N, K)
-    h = (xd @ w1d.t()).bfloat16().float()                        # K.cu:919-931 keeps h in bf16
+    if up_sums is None:
+        w1d = w1_e.float() * _expand_block_scale(w1s_e, N, K)
+        up_sums = xd @ w1d.t()
+    if up_nudge:
+        up_sums = up_sums * (1.0 + up_nudge)
+    h = up_sums.bfloat16().float()                               # K.cu:919-931 keeps h in bf16
     a = _silu_mul(h[:, :I], h[:, I:]).bfloat16().float()         # K.cu:945-946
     n = a.shape[0]
     ag = a.reshape(n, I // 128, 128)
@@ -173,8 +197,20 @@ def _expert_forward(xd, w1_e, w1s_e, w2_e, w2s_e):
 
 
 def fused_moe_oracle(x, x_scale, w, w_scale, w2, w2_scale, sorted_token_ids, expert_ids,
-                     num_tokens_post_padded, topk_weights, out, top_k, block_m, scaling_factor):
+                     num_tokens_post_padded, topk_weights, out, top_k, block_m, scaling_factor, accumulate="dense",
+                     up_nudge=0.0):
     """What torch.ops.alpha_moe.fused_moe_w8a8_up_down leaves in ``out``, computed in fp32 on the CPU.
+
+    accumulate: "dense" sums the up/gate products as one fp32 matrix product of the dequantised operands (the
+    definition every pin of this oracle uses); "kblock" sums them per 128-wide K block and folds the block scales in
+    with fp32 multiply-adds, the order of a block-scaled kernel (_up_sums_kblock) - the same mathematics, used by the
+    tests to tell a legitimate rounding-order difference from an error.
+
+    up_nudge: multiplies every up/gate sum by (1 + up_nudge) before it is rounded to bf16.  The operator is
+    discontinuous in those sums: a sum on a bf16 rounding boundary that is also the largest activation of its
+    128-column group decides the group's FP8 scale, and with it the rounding of all 128 codes.  Sums of thousands of
+    fp32 products accumulated in another order differ by ~1e-5 of their size where terms cancel; a result that agrees
+    with the oracle for some |up_nudge| <= 1e-5 is a result of the same mathematics.
 
     Takes the operator's own arguments (interleaved w / w_scale, routing arrays) and returns a new
     bf16 tensor = out + contribution; ``out`` is not modified.  Walks the routing arrays exactly as the
@@ -204,7 +240,8 @@ def fused_moe_oracle(x, x_scale, w, w_scale, w2, w2_scale, sorted_token_ids, exp
         tok = ids // top_k
         w1_e = deinterleave_reference(w[e:e + 1].view(torch.uint8), 8)[0].view(torch.float8_e4m3fn)
         w1s_e = deinterleave_reference(w_scale[e:e + 1], 1)[0]
-        y = _expert_forward(xd_all[tok], w1_e, w1s_e, w2[e], w2_scale[e])
+        up_sums = _up_sums_kblock(fp8_to_float(x[tok]), x_scale[tok], w1_e, w1s_e) if accumulate == "kblock" else None
+        y = _expert_forward(xd_all[tok], w1_e, w1s_e, w2[e], w2_scale[e], up_sums, up_nudge)
         y = y * (tw_flat[ids] * float(scaling_factor)).unsqueeze(1)            # K.cu:997-1003
         acc.index_add_(0, tok, y)
     return (from_dev(out).float() + acc).bfloat16()

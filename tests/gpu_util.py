@@ -43,14 +43,15 @@ def run_op(P, block_m, block_n, warp_n, stages, out=None, scaling=None, via="tor
     return out
 
 
-def oracle_out(P, block_m=16, out=None, scaling=None):
+def oracle_out(P, block_m=16, out=None, scaling=None, accumulate="dense", up_nudge=0.0):
     W = P.weights
     s_ids, e_ids, total = P.align(block_m)
     if out is None:
         out = torch.zeros((P.M, P.shape.K), dtype=torch.bfloat16)
     scaling = P.shape.scaling_factor if scaling is None else scaling
     return O.fused_moe_oracle(P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids, total,
-                              P.topk_weights, out, P.shape.top_k, block_m, scaling)
+                              P.topk_weights, out, P.shape.top_k, block_m, scaling, accumulate=accumulate,
+                              up_nudge=up_nudge)
 
 
 def assert_parity(out, ref, what=""):
@@ -58,6 +59,29 @@ def assert_parity(out, ref, what=""):
     assert torch.isfinite(out.float()).all(), what
     assert m["max_abs_over_max_ref"] <= MAX_ABS_OVER_MAX_REF and m["cosine"] >= MIN_COSINE, (what, m)
     return m
+
+
+# The operator is discontinuous in its fp32 up/gate sums (bf16 rounding, then an FP8 scale per 128 columns taken from
+# the largest activation): a sum within rounding-order noise of a bf16 boundary may legitimately fall on either side.
+# The oracle recomputed with its sums moved by this relative amount, either way, brackets that noise.
+UP_SUM_NOISE = 1e-5
+
+
+def oracle_variants(P, block_m=16, out=None, scaling=None):
+    """The oracle and its two neighbours within rounding-order noise of the up/gate sums."""
+    return [oracle_out(P, block_m, out, scaling, up_nudge=d) for d in (0.0, UP_SUM_NOISE, -UP_SUM_NOISE)]
+
+
+def assert_parity_rows(out, refs, what=""):
+    """The parity bar per token row against the nearest of `refs` (oracle_variants): every row within 1e-2 of the
+    output range of one of them, and the whole output at cosine >= 0.9999 with the first.  Returns the worst row."""
+    o = out.detach().float().cpu()
+    assert torch.isfinite(o).all(), what
+    scale = refs[0].float().abs().max().clamp_min(1e-30)
+    per_row = torch.stack([(o - r.float()).abs().amax(dim=1) for r in refs]).amin(dim=0) / scale
+    m = O.error_metrics(out, refs[0])
+    assert float(per_row.max()) <= MAX_ABS_OVER_MAX_REF and m["cosine"] >= MIN_COSINE, (what, float(per_row.max()), m)
+    return float(per_row.max())
 
 
 @contextlib.contextmanager
@@ -76,9 +100,28 @@ def tunables(**values):
 def sampled_tokens_match_oracle(P, out, what, n=48, seed=11):
     """A token's result depends on nothing but its own row, routing and the weights: the oracle recomputes a random
     sample of the tokens as an n-token problem of its own."""
+    sub, idx = sample_problem(P, n, seed)
+    return assert_parity(out[idx], oracle_out(sub), what)
+
+
+def sample_problem(P, n, seed):
     from alpha_moe_python.workloads import Problem
     gen = torch.Generator().manual_seed(seed)
     idx = torch.randperm(P.M, generator=gen)[:n].sort().values.to(P.x.device)
-    sub = Problem(P.weights, n, P.x[idx].contiguous(), P.x_scale[idx].contiguous(), P.topk_ids[idx].contiguous(),
+    sub = Problem(P.weights, idx.numel(), P.x[idx].contiguous(), P.x_scale[idx].contiguous(), P.topk_ids[idx].contiguous(),
                   P.topk_weights[idx].contiguous())
-    return assert_parity(out[idx], oracle_out(sub), what)
+    return sub, idx
+
+
+def worst_row_error(P, out, n=None, seed=11):
+    """max |err| / max |ref| of the worst token row (of a sample of n tokens when n is given), against the oracle as it
+    is; where that exceeds the bar, against the nearest of the oracle's neighbours within rounding-order noise of the
+    up/gate sums (assert_parity_rows), which then also checks the bar."""
+    sub, idx = (P, None) if n is None or n >= P.M else sample_problem(P, n, seed)
+    got = out if idx is None else out[idx]
+    ref = oracle_out(sub)
+    m = O.error_metrics(got, ref)
+    assert torch.isfinite(got.float()).all() and m["cosine"] >= MIN_COSINE, m
+    if m["max_abs_over_max_ref"] <= MAX_ABS_OVER_MAX_REF:
+        return m["max_abs_over_max_ref"]
+    return assert_parity_rows(got, oracle_variants(sub), f"M={P.M} sample seed {seed}")

@@ -6,7 +6,8 @@ import pytest
 import torch
 
 from alpha_moe_python.workloads import SHAPES, Shape, make_problem, make_weights
-from gpu_util import assert_parity, oracle_out, run_op, sampled_tokens_match_oracle, tunables
+from gpu_util import (assert_parity, assert_parity_rows, oracle_out, oracle_variants, run_op, sampled_tokens_match_oracle,
+                      tunables, worst_row_error)
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -429,15 +430,9 @@ def test_random_small_shapes_and_knobs():
         P = make_problem(W, M, seed=case)
         print(f"case rnd{case} E={E} top_k={top_k} K={K} I={I} M={M} knobs {(block_m, bn, wn, stages)}", flush=True)
         got = run_op(P, block_m, bn, wn, stages, via="c_abi")
-        # Tiny problems have few terms per output: where the device's and the oracle's fp32 sums of one intermediate
-        # value differ in the last bit and that value sits on an FP8 rounding boundary, it moves by a whole FP8 step
-        # (12.5 %), and an output element dominated by it by a few percent - seen as 1.2e-2 of the output range on one of
-        # these cases, identically from every kernel variant.  The bar here is therefore cosine >= 0.9999 and 2e-2 of
-        # the range (the reference's own test uses atol 2e-2, rtol 1e-1); the benchmark shapes keep the 1e-2 bar.
-        from oracle import moe_oracle as O
-        m = O.error_metrics(got, oracle_out(P))
-        assert torch.isfinite(got.float()).all()
-        assert m["cosine"] >= 0.9999 and m["max_abs_over_max_ref"] <= 2e-2 and m["allclose_2e-2_1e-1"], (case, m)
+        # The 1e-2 bar per token row, against the oracle or one of its neighbours within rounding-order noise of the
+        # up/gate sums: a sum on a bf16 rounding boundary that decides a group's FP8 scale may fall on either side.
+        assert_parity_rows(got, oracle_variants(P), f"rnd{case}")
 
 
 @pytest.mark.parametrize("knobs", [(16, 32, 8, 5), (64, 64, 4, 3)])
@@ -487,7 +482,7 @@ def test_workspace_check_reports_an_expired_wait(c1):
     ws.view(torch.int32)[error_word] = 0
     assert_parity(run_op(P, 16, 32, 8, 5, via="c_abi", workspace=ws), ref, "after clearing the error word")
     # An expiry DURING a launch of the streaming kernel reaches the closing items through the counter they poll: the
-    # waiter adds a high bit to it.  Set from the host here, the bit makes that one launch answer NaN (its closing items
+    # waiter sets a high bit in it (an OR, so the value below is what the kernel produces).  Set from the host here, the bit makes that one launch answer NaN (its closing items
     # do not wait and do not trust what they read); the launch resets the counter, and the next one is clean again.
     down_counter, expired_bit = 32, 1 << 30   # StreamCtl::down_done and kExpiredBit in csrc/moe_common.hpp
     ws.view(torch.int32)[down_counter] = expired_bit
@@ -562,30 +557,51 @@ def test_two_streams_at_once(ds_weights):
 def test_tiny_batches(name, ds_weights, qn_weights):
     """M in {1, 2, 4, 8, 16}: K-split UP items whose partial sums the last arrival adds up (in batches of eight
     splits), on both shards, several knobs, adding and storing, two launches bit for bit; against the oracle.  The 1e-2
-    bar holds on the benchmark sizes; on the sizes in between the bar is the random-shape test's (cosine >= 0.9999,
-    2e-2 of the range): with a dozen routed rows, one intermediate value that lands on the other side of an FP8
-    rounding boundary than the oracle's (its fp32 sums run in another order) moves a whole token by 1.2e-2 of the
-    range - seen at M=2."""
-    from oracle import moe_oracle as O
+    bar holds on every size: on the benchmark sizes against the oracle as it is, on the sizes in between per token row
+    against the oracle or its neighbours within rounding-order noise of the up/gate sums (at M=2 of the DeepSeek-V3
+    shard one up-projection sum of the shared expert, the largest activation of its group, sits 6e-6 of its size from a
+    bf16 rounding boundary; the device's K-split sum falls on the other side, the group's FP8 scale moves by 0.6 %, 12
+    of its 128 codes re-round and that token moves by 1.2e-2 of the output range - see test_an_up_sum_on_a_bf16_boundary)."""
     W = ds_weights if name == "ds" else qn_weights
     benchmark_sizes = (1, 4, 16) if name == "ds" else (1,)
     for M in (1, 2, 4, 8, 16):
         P = make_problem(W, M, seed=20 + M)
         ref = oracle_out(P)
+        variants = None if M in benchmark_sizes else oracle_variants(P)
         for knobs in ((16, 32, 8, 5), (16, 64, 4, 3), (8, 32, 8, 2), (32, 64, 4, 4)):
             print(f"case {name} M={M} knobs {knobs}", flush=True)
             got = run_op(P, *knobs, via="c_abi")
             if M in benchmark_sizes:
                 assert_parity(got, ref, f"{name} M={M} knobs {knobs}")
             else:
-                m = O.error_metrics(got, ref)
-                assert m["cosine"] >= 0.9999 and m["max_abs_over_max_ref"] <= 2e-2, (name, M, knobs, m)
+                assert_parity_rows(got, variants, f"{name} M={M} knobs {knobs}")
             assert torch.equal(got, run_op(P, *knobs, via="c_abi")), (name, M, knobs)
             junk = torch.full((P.M, P.shape.K), float("nan"), dtype=torch.bfloat16, device=DEV)
             assert torch.equal(run_op(P, *knobs, out=junk, via="c_abi", store=True), got), (name, M, knobs, "store")
         pre = torch.full((P.M, P.shape.K), 0.25, dtype=torch.bfloat16, device=DEV)
-        want = O.error_metrics(run_op(P, 16, 32, 8, 5, out=pre.clone(), via="c_abi"), oracle_out(P, out=pre.cpu()))
-        assert want["cosine"] >= 0.9999 and want["max_abs_over_max_ref"] <= 2e-2, (name, M, "out pre-filled", want)
+        assert_parity_rows(run_op(P, 16, 32, 8, 5, out=pre.clone(), via="c_abi"), oracle_variants(P, out=pre.cpu()),
+                           f"{name} M={M} out pre-filled")
+
+
+def test_an_up_sum_on_a_bf16_boundary(ds_weights):
+    """The one problem on which the device and the oracle disagree by more than the bar (DeepSeek-V3 shard, M=2): the
+    disagreement is the oracle's own discontinuity.  Seventeen of the eighteen (token, slot) rows agree; in the shared
+    expert's row of token 0 the up-projection sum of the group's largest activation is -3.429666, at 0.4986 of the way
+    between two bf16 values, and moving the oracle's sums by 1e-5 of their size moves its answer for that token by 1.2e-2
+    of the output range - onto the device's."""
+    from oracle import moe_oracle as O
+    P = make_problem(ds_weights, 2, seed=22)
+    got = run_op(P, 16, 32, 8, 5, via="c_abi")
+    plain, up, down = oracle_variants(P)
+    scale = float(plain.float().abs().max())
+    row = lambda a, b, t: float((a[t].float().cpu() - b[t].float().cpu()).abs().max()) / scale
+    # the oracle against itself, sums moved by 1e-5: token 0 jumps, token 1 does not
+    assert max(row(plain, up, 0), row(plain, down, 0)) > 1e-2
+    assert max(row(plain, up, 1), row(plain, down, 1)) <= 5e-3
+    # the device is within the bar of the neighbour and, on token 1, of the oracle as it is
+    assert min(row(got, up, 0), row(got, down, 0)) <= 5e-3
+    assert row(got, plain, 1) <= 5e-3
+    assert O.error_metrics(got, plain)["cosine"] >= 0.9999
 
 
 def test_tiny_batch_duplicates_padding_and_missing_experts():
@@ -635,6 +651,31 @@ def test_ring_depth_is_clamped_to_what_lds_holds():
         assert_parity(run_op(P, *knobs, via="c_abi"), ref, f"wide knobs {knobs}")
 
 
+def test_eager_calls_of_growing_size_keep_one_scratch_buffer(c1):
+    """The binding's scratch buffer of a stream that only ever runs eager calls: twenty calls of growing size leave ONE
+    buffer alive (replaced buffers go back to the allocator; growth is geometric, so few of the calls reallocate), and
+    the results stay right across the replacements."""
+    P0, _ = c1
+    W = P0.weights
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    sizes, allocations, last = [], 0, 0
+    with torch.cuda.stream(side):
+        for i in range(20):
+            M = 16 + 40 * i
+            Q = make_problem(W, M, seed=100 + i)
+            knobs = (64, 32, 8, 2) if i % 2 else (16, 64, 4, 3)
+            got = run_op(Q, *knobs, via="torch")
+            n_alive, current, retired = torch.ops.alpha_moe.scratch_buffers(Q.x)
+            assert n_alive == 1 and retired == 0, (i, n_alive, retired)
+            allocations += current != last
+            last = current
+            sizes.append(current)
+            if i in (0, 7, 19):
+                assert_parity(got, oracle_out(Q), f"growing sizes, call {i}")
+    assert sizes == sorted(sizes) and allocations <= 10, (sizes, allocations)
+
+
 def test_scratch_regrowth_after_graph_capture(c1):
     """A graph captured on a stream keeps replaying into the scratch buffer the stream had then, also after a larger
     eager call on the same stream made the binding take a bigger buffer; growth DURING capture is refused with an
@@ -676,6 +717,8 @@ def test_scratch_regrowth_after_graph_capture(c1):
         step(big, big_ids, big_out, big_knobs)
         side.synchronize()
         assert torch.equal(big_out, run_op(big, *big_knobs, via="c_abi"))
+        n_alive, _, retired = torch.ops.alpha_moe.scratch_buffers(P.x)
+        assert n_alive == 2 and retired > 0   # the buffer the graph was captured with is kept beside the new one
         # ... and the graph still replays into the one it was captured with
         for _ in range(3):
             out.fill_(7.0)
@@ -759,3 +802,57 @@ def test_prepacked_weights_give_the_same_bits(c1, ds_weights, q3_weights):
     Pf = make_problem(Wf, 8, seed=5)
     with pytest.raises(AssertionError):
         _run_prepacked(Pf, prepack_weights(Wf.w1, Wf.w2), (128, 64, 4, 2))
+
+
+# ---- the reference's correctness sweep on real-K problems, and the shipped tuning tables on several seeds ----------
+def test_every_knob_on_the_deepseek_shard_M32(ds_weights):
+    """test_moe_correctness.py:172-190 of the reference runs every (block_m, block_n/warp_n, stages) it accepts on
+    K = 7168: 56 K blocks, so K-split counts, ring wrap-around, LDS clamps and item sizes differ per knob set.  All 160
+    against one oracle result (the routing arrays depend on block_m, the result does not)."""
+    P = make_problem(ds_weights, 32, seed=41)
+    ref = oracle_out(P)
+    worst = 0.0
+    for knobs in ALL_KNOBS:
+        print(f"case ds M=32 knobs {knobs}", flush=True)
+        worst = max(worst, assert_parity(run_op(P, *knobs, via="c_abi"), ref, f"ds M=32 knobs {knobs}")["max_abs_over_max_ref"])
+    print(f"worst of {len(ALL_KNOBS)} knob sets: {worst:.2e}", flush=True)
+
+
+def test_every_knob_on_a_37_expert_shape_M128():
+    """The reference's sweep shape E = 37, N = 256, K = 4096, shared expert last (test_moe_correctness.py:133,172-190),
+    M = 128: every accepted knob set against one oracle result."""
+    shape = Shape("e37", E=37, top_k=9, K=4096, I=128, shared_expert=True, routing="softmax_shared", scaling_factor=2.5)
+    W = make_weights(shape, device=DEV, seed=37)
+    P = make_problem(W, 128, seed=37)
+    ref = oracle_out(P)
+    worst = 0.0
+    for knobs in ALL_KNOBS:
+        print(f"case e37 M=128 knobs {knobs}", flush=True)
+        worst = max(worst, assert_parity(run_op(P, *knobs, via="c_abi"), ref, f"e37 M=128 knobs {knobs}")["max_abs_over_max_ref"])
+    print(f"worst of {len(ALL_KNOBS)} knob sets: {worst:.2e}", flush=True)
+
+
+SHIPPED = {"ds": ("moe_jit_257_512_7168.json", (1, 4, 16, 64, 512, 2048, 8192)),
+           "qn": ("moe_jit_512_512_2048.json", (1, 32, 256, 4096)),
+           "q3": ("moe_jit_128_1536_2048.json", (64, 1024, 8192))}
+
+
+@pytest.mark.parametrize("name", ["ds", "qn", "q3"])
+def test_shipped_tables_on_four_seeds(name, ds_weights, qn_weights, q3_weights):
+    """Every benchmark size with the knobs the shipped tuning table gives for it (what bench.py and callers run), on
+    four seeds each: the worst token row stays within the bar.  Sizes up to 64 tokens are checked whole, larger ones on
+    a sample of 32 tokens recomputed by the oracle as a problem of their own."""
+    import os
+    from alpha_moe_python.utils import get_best_config
+    table, sizes = SHIPPED[name]
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "alpha-moe_amd", "configs", table)
+    W = {"ds": ds_weights, "qn": qn_weights, "q3": q3_weights}[name]
+    for M in sizes:
+        cfg = get_best_config(path, M)
+        knobs = (cfg["block_m"], cfg["block_n"], cfg["warp_n"], cfg["stages"])
+        worst = 0.0
+        for seed in (101, 102, 103, 104):
+            P = make_problem(W, M, seed=seed)
+            got = run_op(P, *knobs, via="c_abi")
+            worst = max(worst, worst_row_error(P, got, n=32 if M > 64 else None, seed=seed))
+        print(f"{name} M={M} knobs {knobs}: worst row of four seeds {worst:.2e}", flush=True)

@@ -163,3 +163,69 @@ def test_c1_config_runs_and_is_finite():
     assert out.shape == (16, 512) and torch.isfinite(out.float()).all()
     assert 0.01 < float(out.float().abs().max()) < 100
     assert P.algorithmic_flops() == 3 * 16 * 2 * 512 * 256
+
+
+def test_block_scales_land_on_the_right_blocks_exactly():
+    """Power-of-two block scales, every 128x128 weight block and every token group its own, small-integer values: all
+    products and sums stay exact, so the scale of block (row block, K block) is pinned against torch.matmul on weights
+    dequantised explicitly in their ORIGINAL (not interleaved) layout.  A scale row read from the wrong place - gate
+    instead of up, slice b instead of b+1, K block k instead of k+1 - changes the result by a power of two."""
+    g = torch.Generator().manual_seed(7)
+    E, K, I, M, top_k = 2, 384, 256, 5, 2
+    N = 2 * I
+    x = torch.randint(-2, 3, (M, K), generator=g).float()
+    w1o = torch.randint(-1, 2, (E, N, K), generator=g).float()
+    w2 = torch.randint(-2, 3, (E, K, I), generator=g).float()
+    pow2 = lambda *shape: torch.pow(2.0, torch.randint(-3, 4, shape, generator=g).float())
+    xs = pow2(M, K // 128)
+    w1so = pow2(E, N // 128, K // 128)          # original layout: gate row blocks, then up row blocks
+    w2s = pow2(E, K // 128, I // 128)
+    assert len(set(w1so.flatten().tolist())) > 3 and len(set(w2s.flatten().tolist())) > 3
+    ids = torch.stack([torch.randperm(E, generator=g)[:top_k] for _ in range(M)]).to(torch.int32)
+    tw = pow2(M, top_k)
+    block_m = 8
+    s_ids, e_ids, total = moe_align_block_size(ids, block_m, E)
+    got = O.fused_moe_oracle(x.to(torch.float8_e4m3fn), xs, interleave_tensor(w1o.to(torch.float8_e4m3fn), 8),
+                             interleave_tensor(w1so, 1), w2.to(torch.float8_e4m3fn), w2s, s_ids, e_ids, total, tw,
+                             torch.zeros((M, K), dtype=torch.bfloat16), top_k, block_m, 2.0)
+    for accumulate in ("dense", "kblock"):
+        alt = O.fused_moe_oracle(x.to(torch.float8_e4m3fn), xs, interleave_tensor(w1o.to(torch.float8_e4m3fn), 8),
+                                 interleave_tensor(w1so, 1), w2.to(torch.float8_e4m3fn), w2s, s_ids, e_ids, total, tw,
+                                 torch.zeros((M, K), dtype=torch.bfloat16), top_k, block_m, 2.0, accumulate=accumulate)
+        assert torch.equal(alt, got), accumulate        # nothing rounds before the bf16 casts: any order, same bits
+    # the textbook computation on explicitly dequantised weights, no routing arrays
+    xd = x * xs.repeat_interleave(128, dim=1)
+    want = torch.zeros((M, K))
+    for t in range(M):
+        for s in range(top_k):
+            e = int(ids[t, s])
+            w1d = w1o[e] * w1so[e].repeat_interleave(128, 0).repeat_interleave(128, 1)
+            w2d = w2[e] * w2s[e].repeat_interleave(128, 0).repeat_interleave(128, 1)
+            h = (xd[t] @ w1d.t()).bfloat16().float()
+            a = (torch.nn.functional.silu(h[:I]) * h[I:]).bfloat16().float().reshape(I // 128, 128)
+            sa = a.abs().amax(-1, keepdim=True).clamp_min(1e-10) / 448.0
+            q = (a / sa).clamp(-448, 448).to(torch.float8_e4m3fn).float()
+            want[t] += ((q * sa).reshape(I) @ w2d.t()) * float(tw[t, s]) * 2.0
+    m = O.error_metrics(got, want.bfloat16())
+    assert m["max_abs_over_max_ref"] <= 2 ** -8 and float(want.abs().max()) > 1.0, m
+    # the C restatement, which reads the interleaved scale rows 2b / 2b+1 the way the reference kernel does
+    c = c_oracle.fused_moe_c(x.to(torch.float8_e4m3fn), xs, interleave_tensor(w1o.to(torch.float8_e4m3fn), 8),
+                             interleave_tensor(w1so, 1), w2.to(torch.float8_e4m3fn), w2s, s_ids, e_ids, total, tw,
+                             torch.zeros((M, K), dtype=torch.bfloat16), top_k, block_m, 2.0)
+    assert O.error_metrics(c, want.bfloat16())["max_abs_over_max_ref"] <= 2 ** -7
+
+
+def test_accumulation_orders_and_nudged_sums_stay_close():
+    """On ordinary data the K-block-wise accumulation order and sums moved by 1e-5 give the dense oracle's answer to
+    within a bf16 ulp or two of the largest output: they are the same mathematics."""
+    P = _small_problem(E=4, K=512, I=128, M=9, seed=21)
+    s_ids, e_ids, total = P.align(8)
+    W = P.weights
+    run = lambda **kw: O.fused_moe_oracle(P.x, P.x_scale, W.w1, W.w1_scale, W.w2, W.w2_scale, s_ids, e_ids, total,
+                                          P.topk_weights, torch.zeros((P.M, P.shape.K), dtype=torch.bfloat16),
+                                          P.shape.top_k, 8, P.shape.scaling_factor, **kw)
+    base = run()
+    for kw in ({"accumulate": "kblock"}, {"up_nudge": 1e-5}, {"up_nudge": -1e-5}):
+        m = O.error_metrics(run(**kw), base)
+        assert m["max_abs_over_max_ref"] <= 1e-2 and m["cosine"] >= 0.9999, (kw, m)
+    assert torch.equal(run(up_nudge=0.0), base)
