@@ -146,37 +146,35 @@ __device__ __forceinline__ void lds_barrier()
 }
 
 // Agent-scope (sc1) accesses for data that crosses workgroups - and XCDs, whose L2s are not coherent with each other -
-// inside one launch.  The asm ones are invisible to the compiler's wait-count insertion: drain_vmem_into() the
-// registers they load before using them, drain_vmem() before telling anybody about what they stored.
-__device__ __forceinline__ v4i ldg128_agent(const void *p)
+// inside one launch.  The 16- and 4-byte ones are raw buffer operations on a buffer that starts at a wavefront-uniform
+// base and has no end, addressed by a 32-bit per-lane byte offset: the cache-policy bits are an argument of the builtin
+// (no flat or global builtin takes them), and unlike inline asm the compiler sees these accesses - it places the wait
+// before the first use of a loaded register, keeps that register live until then, and honours the hazard between a
+// wide store and the next write of its data registers.  drain_vmem() before telling anybody about what was stored;
+// acquire_fence() between seeing another workgroup's flag and loading what it published.
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+constexpr int kAuxAgent = 16;   // sc1
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t agent_buffer(const void *uniform_base)
 {
-    v4i r;
-    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=v"(r) : "v"(p) : "memory");
-    return r;
+    const uint64_t v = reinterpret_cast<uint64_t>(uniform_base);
+    const uint64_t u = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32)) << 32) |
+                       (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void *>(u), 0, -1, 0x00020000);
 }
-// Wait for everything this wavefront has in flight and hand the registers of up to eight ldg128_agent() loads over
-// to the compiler only now: as in/out operands of the wait they cannot be read - and their registers cannot be given
-// to anything else - before the data has landed.  (A bare wait would not do: the compiler sees an asm load's result as
-// ready at once, and a late-landing load then overwrites whatever it moved into those registers, addresses included.)
-__device__ __forceinline__ void drain_vmem_into(v4i (&r)[8])
+__device__ __forceinline__ v4i ldg128_agent(const void *uniform_base, uint32_t byte_off)
 {
-    asm volatile("s_waitcnt vmcnt(0)"
-                 : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7])
-                 :
-                 : "memory");
-    __builtin_amdgcn_sched_barrier(0);
+    return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(agent_buffer(uniform_base), (int)byte_off, 0, kAuxAgent));
 }
-__device__ __forceinline__ void stg32_agent(void *p, uint32_t v)
+__device__ __forceinline__ void stg32_agent(void *uniform_base, uint32_t byte_off, uint32_t v)
 {
-    asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    __builtin_amdgcn_raw_buffer_store_b32(v, agent_buffer(uniform_base), (int)byte_off, 0, kAuxAgent);
 }
-__device__ __forceinline__ void stg128_agent(void *p, v4f v)
+__device__ __forceinline__ void stg128_agent(void *uniform_base, uint32_t byte_off, v4f v)
 {
-    // The hardware reads the data registers of a store wider than 64 bits a few cycles after issue; the compiler's
-    // hazard recognizer cannot see into inline asm, so the wait states before those registers may be overwritten
-    // are spelled out here.
-    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 2" ::"v"(p), "v"(v) : "memory");
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), agent_buffer(uniform_base), (int)byte_off, 0, kAuxAgent);
 }
+// nothing that reads memory may be moved by the compiler from behind this point to before it
+__device__ __forceinline__ void acquire_fence() { asm volatile("" ::: "memory"); }
 __device__ __forceinline__ int load_agent(const int *p)
 {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -238,7 +236,10 @@ __device__ __noinline__ inline void spin_all_ge(const int *addr, int count, int 
     const int lane = threadIdx.x & 63;
     for (int it = 0; it < (1 << 22); it++) {
         const int v = lane < count ? load_agent(addr + lane) : target;
-        if (__all(reached(v, target))) return;
+        if (__all(reached(v, target))) {
+            acquire_fence();
+            return;
+        }
         if (it < 16) __builtin_amdgcn_s_sleep(4);
         else __builtin_amdgcn_s_sleep(32);
     }

@@ -200,10 +200,10 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                     pack_fp8x4(clamp_fp8(accg[pr][t][0] / s_a), clamp_fp8(accg[pr][t][1] / s_a),
                                clamp_fp8(accg[pr][t][2] / s_a), clamp_fp8(accg[pr][t][3] / s_a));
                 const int col = wave * (RW / 2) + pr * 16 + 4 * q;
-                stg32_agent(aq_u + (t * 16 + n) * 128 + col, packed);
+                stg32_agent(aq_u, (uint32_t)((t * 16 + n) * 128 + col), packed);
             }
             if (wave == 0 && q == 0)
-                stg32_agent(&s.sa[(size_t)u * s.bm_pad + t * 16 + n], __builtin_bit_cast(uint32_t, s_a));
+                stg32_agent(s.sa + (size_t)u * s.bm_pad, (uint32_t)(t * 16 + n) * 4u, __builtin_bit_cast(uint32_t, s_a));
         }
         drain_vmem();
         __syncthreads();
@@ -344,9 +344,9 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 if (!r.valid[t]) continue;
 #pragma unroll
                 for (int pr = 0; pr < NP; pr++) {
-                    float *dst = h_u + ksp * slice + t * 16 * 256 + my_off + pr * 16;
-                    stg128_agent(dst, accg[pr][t]);
-                    stg128_agent(dst + 128, accu[pr][t]);
+                    const uint32_t off = (uint32_t)(t * 16 * 256 + my_off + pr * 16) * 4u;
+                    stg128_agent(h_u + ksp * slice, off, accg[pr][t]);
+                    stg128_agent(h_u + ksp * slice, off + 512u, accu[pr][t]);
                 }
             }
             drain_vmem();
@@ -355,6 +355,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 s_bcast[1] = __hip_atomic_fetch_add(&s.arrive[u], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             __syncthreads();
             if (s_bcast[1] != s.ks - 1) return;
+            acquire_fence();   // the other splits' partial sums are read from here on, not before
             if (tid == 0) store_agent(&s.arrive[u], 0);
 #pragma unroll
             for (int t = 0; t < TM; t++)
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 for (int pr = 0; pr < NP; pr++) {
                     v4f g = {0.f, 0.f, 0.f, 0.f}, up = {0.f, 0.f, 0.f, 0.f};
                     if (r.valid[t]) {
-                        const float *src = h_u + t * 16 * 256 + my_off + pr * 16;
+                        const uint32_t off = (uint32_t)(t * 16 * 256 + my_off + pr * 16) * 4u;
                         // fixed order: the sum does not depend on arrival order.  Eight splits (16 loads) are in flight
                         // at a time: one memory round trip per batch, not per split.
                         for (int k0 = 0; k0 < s.ks; k0 += 8) {
@@ -370,11 +371,9 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
 #pragma unroll
                             for (int k = 0; k < 8; k++) {
                                 const int kk = k0 + k < s.ks ? k0 + k : s.ks - 1;
-                                gk[k] = ldg128_agent(src + kk * slice);
-                                uk[k] = ldg128_agent(src + kk * slice + 128);
+                                gk[k] = ldg128_agent(h_u + kk * slice, off);
+                                uk[k] = ldg128_agent(h_u + kk * slice, off + 512u);
                             }
-                            drain_vmem_into(gk);
-                            drain_vmem_into(uk);
 #pragma unroll
                             for (int k = 0; k < 8; k++)
                                 if (k0 + k < s.ks) {
@@ -470,11 +469,11 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                     sa_bits[k] = load_agent(reinterpret_cast<const int *>(&s.sa[(size_t)(mb * n_ib + ib) * s.bm_pad + row]));
             }
             float tw[TM];
-            float *yp[TM];
+            uint32_t yoff[TM];   // byte offset of this lane's 4 columns in the slot's row of y (rows * K * 4 <= 2^30)
 #pragma unroll
             for (int t = 0; t < TM; t++) {
                 tw[t] = r.valid[t] ? p.topk_w[r.slot[t]] * p.scaling : 0.f;
-                yp[t] = s.y + (size_t)r.slot[t] * K + 4 * q;
+                yoff[t] = ((uint32_t)r.slot[t] * (uint32_t)K + 4u * q) * 4u;
                 if (cs == 0 && wave == 0 && q == 0 && r.valid[t]) store_agent(&s.live[r.slot[t]], epoch);
             }
 #pragma unroll
@@ -530,7 +529,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                     if (g0 + gg < wng) {
 #pragma unroll
                         for (int t = 0; t < TM; t++)
-                            if (r.valid[t]) stg128_agent(yp[t] + ((wt0 + g0 + gg) << 4), res[gg][t]);
+                            if (r.valid[t]) stg128_agent(s.y, yoff[t] + ((uint32_t)(wt0 + g0 + gg) << 6), res[gg][t]);
                     }
             }
         }
@@ -566,6 +565,7 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
             }
         }
         __syncthreads();
+        acquire_fence();   // the result rows are read from here on, not before the DOWN counter was seen up
         // an item sums fin_w (1 or 2) chunks of 1024 columns: with more chunks than workgroups, two per item halve the
         // rounds of dependent memory round trips that close the call
         const bool poisoned = s_bcast[1] != 0;
@@ -597,15 +597,10 @@ __global__ __launch_bounds__(WN * 64) void moe_stream_kernel(const StreamPlan s)
                 for (int k = 0; k < 8; k++) {
                     lo[j][k] = (v4i){0, 0, 0, 0};
                     hi[j][k] = (v4i){0, 0, 0, 0};
-                    const float *row = s.y + (size_t)(tk[j] * p.top_k + s0 + k) * K + col[j];
-                    if (mine[j] && s0 + k < p.top_k) lo[j][k] = ldg128_agent(row);
-                    if (mine[j] && s0 + 8 + k < p.top_k) hi[j][k] = ldg128_agent(row + (size_t)8 * K);
+                    const uint32_t row = ((uint32_t)(tk[j] * p.top_k + s0 + k) * (uint32_t)K + (uint32_t)col[j]) * 4u;
+                    if (mine[j] && s0 + k < p.top_k) lo[j][k] = ldg128_agent(s.y, row);
+                    if (mine[j] && s0 + 8 + k < p.top_k) hi[j][k] = ldg128_agent(s.y, row + 32u * (uint32_t)K);
                 }
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                drain_vmem_into(lo[j]);
-                drain_vmem_into(hi[j]);
-            }
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 const unsigned long long live_mask = __ballot(lane < p.top_k && stamp[j] == epoch) >> s0;

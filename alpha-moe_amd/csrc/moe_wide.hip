@@ -512,9 +512,9 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
                             pack_fp8x4(clamp_fp8(acc[2 * pr][t][0] / s_a), clamp_fp8(acc[2 * pr][t][1] / s_a),
                                        clamp_fp8(acc[2 * pr][t][2] / s_a), clamp_fp8(acc[2 * pr][t][3] / s_a));
                         // columns w*32 + pr*16 + 4q .. +3 of token n: chunk w*2 + pr of the row, bytes 4q .. 4q+3 in it
-                        stg32_agent(tile + n * 128 + 16 * ((w * 2 + pr) ^ f_n) + 4 * q, packed);
+                        stg32_agent(tile, (uint32_t)(n * 128 + 16 * ((w * 2 + pr) ^ f_n) + 4 * q), packed);
                     }
-                    if (w == 0 && q == 0) stg32_agent(&s.sas[gt * 16 + n], __builtin_bit_cast(uint32_t, s_a));
+                    if (w == 0 && q == 0) stg32_agent(s.sas + gt * 16, 4u * n, __builtin_bit_cast(uint32_t, s_a));
                 }
             }
             wait_vmcnt<0>();
