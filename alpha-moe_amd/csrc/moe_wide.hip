@@ -51,7 +51,8 @@ struct WideParams {
     uint16_t *y;      // [slots][K] bf16
     uint8_t *aqs;     // [n_ib][n_tiles_total] requantised operand tiles of 2 KiB
     float *sas;       // [n_ib][n_tiles_total * 16] their per-token scales
-    int *plan;        // [0] macro blocks of this launch, [1 + m] first row block of macro block m
+    int *plan;        // [0] macro blocks of this launch; [4 + 4 m ..]: first row block, expert, row blocks, "the expert's
+                      // only macro block" of macro block m
     int n_ib, nkb, n_mb_max;
     int blocks_per_macro;   // floor(256 / block_m)
     int tpb;                // 16-row tile slots per row block in scratch, ceil(block_m / 16)
@@ -129,7 +130,13 @@ __global__ __launch_bounds__(1024) void moe_wide_plan_kernel(const WideParams s)
         __syncthreads();
         int pos = s_carry[1] + __builtin_popcountll(lmask & ((1ull << lane) - 1ull));
         for (int v = 0; v < wave; v++) pos += s_count[v];
-        if (leader) s.plan[1 + pos] = mb;
+        if (leader) {
+            // the macro block's row blocks: up to blocks_per_macro consecutive ones of this expert
+            int nb = 1;
+            while (nb < s.blocks_per_macro && mb + nb < n_live && p.expert_ids[mb + nb] == e) nb++;
+            const bool more_after = mb + nb < n_live && p.expert_ids[mb + nb] == e;
+            *reinterpret_cast<v4i *>(&s.plan[4 + 4 * pos]) = (v4i){mb, e, nb, (mb == start && !more_after) ? 1 : 0};
+        }
         __syncthreads();
         if (tid == 1023) {
             int total = pos + (leader ? 1 : 0);
@@ -318,18 +325,15 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
         int mb0, e, row0, n_rows;
         bool lone;   // the expert has no other macro block
     };
-    auto macro_of = [&](int m) {
+    auto macro_of = [&](int m) {   // one load: the plan kernel has looked the expert ids up
+        const v4i ent = *reinterpret_cast<const v4i *>(&s.plan[4 + 4 * m]);
         Macro mc;
-        mc.mb0 = rfl(s.plan[1 + m]);
-        mc.e = rfl(p.expert_ids[mc.mb0]);
-        int nb = 1;
-        while (nb < s.blocks_per_macro && mc.mb0 + nb < n_live && rfl(p.expert_ids[mc.mb0 + nb]) == mc.e) nb++;
+        mc.mb0 = rfl(ent.x);
+        mc.e = rfl(ent.y);
         mc.row0 = mc.mb0 * p.block_m;
-        mc.n_rows = nb * p.block_m;
+        mc.n_rows = rfl(ent.z) * p.block_m;
         if (mc.row0 + mc.n_rows > p.sorted_num) mc.n_rows = p.sorted_num - mc.row0;
-        const bool left = mc.mb0 > 0 && rfl(p.expert_ids[mc.mb0 - 1]) == mc.e;
-        const bool right = mc.mb0 + nb < n_live && rfl(p.expert_ids[mc.mb0 + nb]) == mc.e;
-        mc.lone = s.w_nt >= 0 ? s.w_nt != 0 : (!left && !right);
+        mc.lone = s.w_nt >= 0 ? s.w_nt != 0 : rfl(ent.w) != 0;
         return mc;
     };
     // Routing of the block's rows into LDS; returns the number of 16-row tiles up to the last valid row.
@@ -797,7 +801,7 @@ size_t wide_workspace_bytes(int top_k, int M, int K, int N, int E, int sorted_nu
     const size_t tiles = n_mb * ((block_m + 15) / 16);
     return align_up(kPrefixBytes) + align_up((size_t)M * top_k * K * sizeof(uint16_t)) +
            align_up((size_t)(N / 256) * tiles * 2048) + align_up((size_t)(N / 256) * tiles * 16 * sizeof(float)) +
-           align_up((n_mb + 1) * sizeof(int));
+           align_up((n_mb + 1) * 4 * sizeof(int));
 }
 
 hipError_t launch_wide(const MoeParams &p, int stages, void *workspace, hipStream_t stream)

@@ -29,12 +29,21 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.join(ROOT, "alpha-moe_amd"))
 sys.path.insert(0, ROOT)
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy of known size), for the
-# configurations that were profiled (all kernels of a call):
-#   profiles/moe_stream_kernel_ds_decode_M64_hbm_traffic.md, profiles/moe_tile_kernel_ds_prefill_M8192_hbm_traffic.md,
-#   profiles/moe_tile_kernel_q3_prefill_M8192_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES = {("ds", 64): 1293.5e6, ("ds", 512): 1676.0e6, ("ds", 2048): 2240.8e6, ("ds", 8192): 4802.9e6,
-                          ("q3", 1024): 813.4e6, ("q3", 8192): 1897.0e6}
+# HBM bytes per call from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by a copy of known size; all kernels of a
+# call) live in profiles/traffic.json together with the library version they were measured on: a build of another
+# version reports null instead of a stale figure.
+def load_measured_traffic(library_version):
+    path = os.path.join(ROOT, "profiles", "traffic.json")
+    try:
+        with open(path) as f:
+            doc = json.load(f)
+    except (OSError, ValueError):
+        return {}
+    if doc.get("library_version") != library_version:
+        return {}
+    return {tuple(k.split("/")[:1]) + (int(k.split("/")[1]),): float(v) for k, v in doc.get("bytes_per_call", {}).items()}
+
+
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 FP8_PEAK_TFLOPS = 5000.0     # MI355X dense FP8 MFMA, published
 DEFAULT_KNOBS = {"block_m": 16, "block_n": 32, "warp_n": 8, "stages": 5}
@@ -73,7 +82,8 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         return 2
-    import alpha_moe  # noqa: F401  fails loudly if the HIP libraries are not built
+    import alpha_moe  # fails loudly if the HIP libraries are not built
+    MEASURED_TRAFFIC_BYTES = load_measured_traffic(alpha_moe.__version__)
     from alpha_moe_python.utils import get_best_config
     from alpha_moe_python.workloads import SHAPES, Weights, make_problem, make_weights
 
@@ -240,20 +250,24 @@ def main():
     per_M = dict(sorted(per_M.items(), key=lambda kv: int(kv[0])))
 
     achieved = head["bytes"] / head["launch_us_mean"] / 1e3   # GB/s
-    knobs_bm = head["knobs"]["block_m"]
+
+    def kernel_of(knobs):
+        if knobs["block_m"] <= 32:
+            return "moe_stream_kernel"
+        return "moe_wide_kernel" if knobs["warp_n"] == 8 else "moe_tile_kernel"
     if args.M >= 4096:   # prefill: the contraction is the bound (the weights stream once; from M ~ 8k the matrix time exceeds the HBM time)
         tflops = head["flops"] / head["launch_us_mean"] / 1e6
         roofline = {"bound": "mfma", "achieved": round(tflops, 1), "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(tflops / FP8_PEAK_TFLOPS, 4),
                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.shape, args.M)),
-                    "kernel": "moe_tile_kernel" if knobs_bm > 32 else "moe_stream_kernel",
+                    "kernel": kernel_of(head["knobs"]),
                     "algorithmic_flops_per_launch": int(head["flops"]),
                     "launch_us_mean": round(head["launch_us_mean"], 2)}
     else:
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBS, 4),
                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.shape, args.M)),
-                    "kernel": "moe_tile_kernel" if knobs_bm > 32 else "moe_stream_kernel",
+                    "kernel": kernel_of(head["knobs"]),
                     "algorithmic_bytes_per_launch": int(head["bytes"]),
                     "launch_us_mean": round(head["launch_us_mean"], 2)}
     result = {
@@ -275,6 +289,19 @@ def main():
         "roofline": roofline,
         "per_M": per_M,
     }
+    # the other half of the metric: the largest prefill size against the FP8 matrix peak (and against the binding bound:
+    # the larger of the algorithmic HBM time and the algorithmic matrix time over the measured time)
+    big = str(max(int(k) for k in per_M))
+    if int(big) >= 4096 and int(big) != args.M:
+        r = per_M[big]
+        t_us = r["launch_us_mean"]
+        t_hbm = r["algorithmic_MB"] * 1e6 / (HBM_PEAK_GBS * 1e9) * 1e6
+        t_mfma = r["TFLOP_per_s"] * t_us / FP8_PEAK_TFLOPS
+        result["roofline_prefill"] = {
+            "workload": f"{shape.name}_prefill_M{big}", "bound": "mfma", "achieved": r["TFLOP_per_s"],
+            "peak": FP8_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": r["mfma_frac"], "hbm_frac": r["hbm_frac"],
+            "binding_frac": round(max(t_hbm, t_mfma) / t_us, 4), "traffic": MEASURED_TRAFFIC_BYTES.get((args.shape, int(big))),
+            "kernel": kernel_of(r["knobs"]), "launch_us_mean": t_us}
 
     if not args.no_cpu_baseline:
         # the CPU port of the reference maths on the same bits, on this box's host cores (checker, not product)
