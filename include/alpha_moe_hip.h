@@ -119,8 +119,8 @@ int alpha_moe_fused_moe_w8a8_up_down_prepacked(
  * ALPHA_MOE_STATIC_SCRATCH_BYTES built into the library's code object (every device the library runs on holds its own
  * copy until the process ends).  The call allocates and frees nothing.  A call whose alpha_moe_workspace_bytes()
  * exceeds that size returns ALPHA_MOE_ERR_SCRATCH_LIMIT and launches nothing: 64 MiB cover every decode-sized batch of
- * the shipped shard shapes (DeepSeek-V3 shard with the shipped knobs: up to M = 256) but not prefill, whose scratch
- * grows with M * top_k * K.  All calls on one device share the one
+ * the shipped shard shapes (DeepSeek-V3 shard with the shipped knobs: up to M = 128, and M = 256 with 16-row blocks;
+ * the other two shards up to M = 1024) but not prefill, whose scratch grows with M * top_k * K.  All calls on one device share the one
  * buffer, which keeps the last call's contents: calls that overlap in time on one device race (order them on one
  * stream), and a bounded wait that ran out stays recorded (every later call then fills `out` with NaN) until
  * alpha_moe_static_scratch_reset clears it.  The first call on a device looks the buffer's address up; make that call outside graph capture.
