@@ -60,6 +60,8 @@ struct WideParams {
     int gps, n_cs;          // 64-column groups per DOWN item, column slabs per macro block
     int lag;                // macro blocks whose up/gate items precede the first down items of a queue
     int w_nt;               // weights with non-temporal loads: 1 always, 0 never, -1 for experts with one macro block
+    int xs_chunk;           // 1: a token's activation scales are fetched four K steps at a time (K / 128 a multiple of 4,
+                            // x_scale 16-byte aligned), 0: one step at a time
 };
 
 __device__ __forceinline__ int rfl(int v) { return __builtin_amdgcn_readfirstlane(v); }
@@ -200,14 +202,16 @@ __device__ __forceinline__ void wide_step(const uint8_t *a_tiles, const uint8_t 
 
 // Half a step: token tiles T0 .. T0 + 3 of the wavefront against weight fragments already in registers.  Same
 // arithmetic and order as wide_step.
+// The per-token factor of the wavefront's token tile t is row[t * row_a + (t >= 4 ? row_b : 0)].
 template <int T0, typename Issue>
-__device__ __forceinline__ void wide_half(const v8i (&a)[4], const uint8_t *b_tiles, const float *row, float sc0,
-                                          float sc1, v4f (&acc)[4][8], int frag_lo, int frag_hi, int nt_w, Issue issue)
+__device__ __forceinline__ void wide_half(const v8i (&a)[4], const uint8_t *b_tiles, const float *row, int row_a, int row_b,
+                                          float sc0, float sc1, v4f (&acc)[4][8], int frag_lo, int frag_hi, int nt_w,
+                                          Issue issue)
 {
     auto read_tile = [&](const uint8_t *tile) -> v8i {
         return cat(*reinterpret_cast<const v4i *>(tile + frag_lo), *reinterpret_cast<const v4i *>(tile + frag_hi));
     };
-    auto row_at = [&](int t) { return row[t < 4 ? t * 64 : (t - 4) * 64 + 16]; };
+    auto row_at = [&](int t) { return row[t * row_a + (t >= 4 ? row_b : 0)]; };
     v8i b = read_tile(b_tiles + T0 * 4096);
     float f = row_at(T0);
 #pragma unroll
@@ -273,6 +277,7 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
     // tiles [n_ib][16] of a resident DOWN item in the same place
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds_dyn[];
     __shared__ float s_xs[2][kWRows];        // per-token factors of a ring stage, tile tt at (tt & 7) * 32 + (tt >> 3) * 16
+    __shared__ __attribute__((aligned(16))) float s_xc[2][kWRows * 4];   // UP, chunked: [chunk & 1][tile][token][step & 3]
     __shared__ float s_ws[2][kWMaxKb];
     __shared__ float s_amax[4][kWRows];
     __shared__ float s_w2s[kWMaxW2s];
@@ -376,6 +381,8 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
         const int unit = mc.mb0 * n_ib + ib;
         if (n_tiles > 0) {
             // token-tile gather: wavefront v loads tiles v and v + 8
+            const bool xs_chunk = s.xs_chunk != 0;
+            const int row_a = xs_chunk ? 128 : 64, row_b = xs_chunk ? 0 : -240;
             unsigned x_off[2][2], xs_off[2];
 #pragma unroll
             for (int j = 0; j < 2; j++)
@@ -420,6 +427,10 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
                 if (i < 2) {
                     dma16_sv<0>(p.x + (size_t)kb * 128, x_off[j][i],
                                 xbuf + stage * kWStageX + (wave + 8 * j) * 2048 + i * 1024);
+                } else if (xs_chunk) {
+                    // steps kb .. kb + 3 of the tile's 16 tokens, 16 bytes per token, with the loads of step kb & ~3
+                    if (kb & 3) return;
+                    if (lane < 16) dma16_sv<0>(p.x_scale + kb, xs_off[j] * 4u, &s_xc[(kb >> 2) & 1][(wave + 8 * j) * 64]);
                 } else if (lane < 16) {
                     dma4_sv<0>(p.x_scale + kb, xs_off[j] * 4u, &s_xs[stage][wave * 32 + 16 * j]);
                 }
@@ -462,18 +473,28 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
                         wait_pending(issued - mark_lo[h]);
                         lds_barrier();   // weight fragments are in registers everywhere; token tiles 0..7 have landed
                         const float sc0 = s_ws[0][kb], sc1 = s_ws[1][kb];
-                        wide_half<0>(a, xbuf + h * kWStageX + g * 2048, &s_xs[h][row_off], sc0, sc1, acc, frag_lo,
+                        const float *row = xs_chunk ? &s_xc[(kb >> 2) & 1][g * 64 + n * 4 + (kb & 3)] : &s_xs[h][row_off];
+                        // loads of the step, five or so per half: weights of step kb + 2 (halves 0, 1 | 2, 3), the
+                        // second token half of step kb + 1 | the first token half of step kb + 2
+                        wide_half<0>(a, xbuf + h * kWStageX + g * 2048, row, row_a, row_b, sc0, sc1, acc, frag_lo,
                                      frag_hi, nt_w, [&](int t) {
-                                         if (kb + 2 < nkb) issue_a_op(kb + 2, h, t);
-                                         if (kb + 1 < nkb && t < 3) issue_x_op(kb + 1, h ^ 1, 1, t);
+                                         if (kb + 2 < nkb && (t & 1) == 0) issue_a_op(kb + 2, h, t >> 1);
+                                         if (kb + 1 < nkb) {
+                                             if (t & 1) issue_x_op(kb + 1, h ^ 1, 1, t >> 1);
+                                             if (t == 3) issue_x_op(kb + 1, h ^ 1, 1, 2);
+                                         }
                                      });
-                        mark_a[h] = issued;        // (a load of step kb + 1's second half may follow the last weight
-                        mark_hi[h ^ 1] = issued;   //  load: waiting for one more than needed is harmless)
+                        mark_hi[h ^ 1] = issued;
                         wait_pending(issued - mark_hi[h]);
                         lds_barrier();   // everybody is done with token tiles 0..7; tiles 8..15 have landed
-                        wide_half<4>(a, xbuf + h * kWStageX + g * 2048, &s_xs[h][row_off], sc0, sc1, acc, frag_lo,
+                        wide_half<4>(a, xbuf + h * kWStageX + g * 2048, row, row_a, row_b, sc0, sc1, acc, frag_lo,
                                      frag_hi, nt_w, [&](int t) {
-                                         if (kb + 2 < nkb && t < 7) issue_x_op(kb + 2, h, 0, t - 4);
+                                         if (kb + 2 < nkb) {
+                                             if ((t & 1) == 0) issue_a_op(kb + 2, h, 2 + ((t - 4) >> 1));
+                                             if (t == 6) mark_a[h] = issued;
+                                             if (t & 1) issue_x_op(kb + 2, h, 0, (t - 4) >> 1);
+                                             if (t == 7) issue_x_op(kb + 2, h, 0, 2);
+                                         }
                                      });
                         mark_lo[h] = issued;
                     }
@@ -830,6 +851,7 @@ hipError_t launch_wide(const MoeParams &p, int stages, void *workspace, hipStrea
     s.n_cs = ((p.K >> 6) + s.gps - 1) / s.gps;
     s.lag = tunable(kTunTileLag, 32);
     s.w_nt = tunable(kTunTileNt, -1);
+    s.xs_chunk = (s.nkb % 4 == 0 && reinterpret_cast<uintptr_t>(p.x_scale) % 16 == 0) ? 1 : 0;
     if (s.lag < 1) s.lag = 1;
     hipError_t err = allow_dynamic_lds();
     if (err != hipSuccess) return err;
