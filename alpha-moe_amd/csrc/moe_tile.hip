@@ -61,6 +61,8 @@ struct TileParams {
     int nh;           // token parts per column slab (a DOWN item is one part of one slab)
     int lag;          // row blocks whose up/gate items precede the first down items of a queue
     int w_nt;         // weights with non-temporal loads: 1 always, 0 never, -1 for experts with a single row block
+    int xs_chunk;     // 1: a token's activation scales are fetched four K steps at a time (K / 128 a multiple of 4,
+                      // x_scale 16-byte aligned), 0: one step at a time
 };
 
 // One step of a wavefront: 4 weight tiles x TH token tiles, all from LDS.  acc[k][t] += (A_k x B_t) * row[t] * sc[k & 1]
@@ -68,9 +70,10 @@ struct TileParams {
 // (k, t) is scaled into its accumulator behind the matrix instruction of (k, t + 1).
 // The step's NOPS direct-to-LDS loads (issue(i), i < NOPS) are spread evenly between the 4 TH matrix instructions: a
 // load instruction blocks its wavefront for 30-60 ns (measured), and the other wavefront of the SIMD computes then.
+// The factor of token tile t is row[t * row_stride].
 template <int TH, int NOPS, typename Issue>
-__device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *b_tiles, const float *row, float sc0,
-                                         float sc1, v4f (&acc)[4][TH], int frag_lo, int frag_hi, Issue issue)
+__device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *b_tiles, const float *row, int row_stride,
+                                         float sc0, float sc1, v4f (&acc)[4][TH], int frag_lo, int frag_hi, Issue issue)
 {
     constexpr int GROUPS = 4 * TH;
     auto read_tile = [&](const uint8_t *tile) -> v8i {
@@ -89,7 +92,7 @@ __device__ __forceinline__ void mma_step(const uint8_t *a_tiles, const uint8_t *
         float f_next = f;
         if (t + 1 < TH) {
             b_next = read_tile(b_tiles + (t + 1) * 2048);
-            f_next = row[(t + 1) * 16];
+            f_next = row[(t + 1) * row_stride];
         }
         v4f cur[4];
 #pragma unroll
@@ -131,11 +134,15 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
     // [4 pairs][3 stages][4 tiles] weight rings | UP items: [3 stages][TM] token tiles; DOWN items: the requantised
     // tiles [n_ib][TM] in the same place
     extern __shared__ __attribute__((aligned(1024))) uint8_t lds_dyn[];
-    __shared__ __attribute__((aligned(1024))) uint8_t s_dummy[2048 + 64];
+    __shared__ __attribute__((aligned(1024))) uint8_t s_dummy[2048 + 256];
     __shared__ float s_xs[kStages][TM * 16];
     __shared__ float s_ws[2][kTileMaxKb];
     __shared__ float s_amax[4][TM * 16];
-    __shared__ float s_sa[kTileMaxIb][TM * 16];
+    __shared__ __attribute__((aligned(16))) float s_sa[kTileMaxIb][TM * 16];
+    // chunked activation scales of UP items, [chunk & 1][tile][token][step & 3], in the place of the DOWN items' s_sa:
+    // items of the two kinds never overlap in a workgroup (a barrier separates them, and an item's loads have landed)
+    static_assert(kTileMaxIb * 16 >= 2 * 64, "s_xc does not fit s_sa");
+    float (*s_xc)[TM * 64] = reinterpret_cast<float (*)[TM * 64]>(&s_sa[0][0]);
     __shared__ float s_w2s[kTileMaxW2s];
     __shared__ int s_tok[TM * 16];
     __shared__ int s_item[2];
@@ -184,6 +191,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
         return !left && !right;
     };
 
+    const bool xs_chunk = s.xs_chunk != 0;
     auto up_item = [&](int mb, int ib) {
         int e = __builtin_amdgcn_readfirstlane(p.expert_ids[mb]);
         if (e < 0 || e >= p.E) return;
@@ -226,11 +234,17 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
                 const int part = i - AOPS;
                 uint8_t *dst = x_real ? xbuf + stage * (TM * 2048) + wave * 2048 : s_dummy;
                 dma16<0>(gx[part] + (size_t)kc * 128, dst + part * 1024);
+            } else if (xs_chunk) {
+                // steps kb .. kb + 3 of the tile's 16 tokens, 16 bytes per token, with the loads of step kb & ~3
+                float *sdst = x_real ? &s_xc[(kb >> 2) & 1][wave * 64] : reinterpret_cast<float *>(s_dummy + 2048);
+                if ((kb & 3) == 0 && lane < 16) dma16<0>(reinterpret_cast<const uint8_t *>(gxs + (kb < nkb ? kb : nkb - 4)), reinterpret_cast<uint8_t *>(sdst));
             } else {
                 float *sdst = x_real ? &s_xs[stage][wave * 16] : reinterpret_cast<float *>(s_dummy + 2048);
                 if (lane < 16) dma4(gxs + kc, sdst);
             }
         };
+        // load instructions of step kb: the scales come with every fourth step when they are fetched in chunks
+        auto ops_of = [&](int kb) { return xs_chunk ? OPS1 - 1 + ((kb & 3) == 0 ? 1 : 0) : OPS1; };
         auto issue_all = [&](int kb, int stage) {
 #pragma unroll
             for (int i = 0; i < OPS1; i++) issue_op(kb, stage, i);
@@ -250,10 +264,13 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
             for (int h = 0; h < kStages; h++) {
                 const int kb = kb0 + h;
                 if (kb < nkb) {
-                    wait_vmcnt<OPS1>();
+                    if (ops_of(kb + 1) == OPS1) wait_vmcnt<OPS1>();
+                    else wait_vmcnt<OPS1 - 1>();
                     lds_barrier();
-                    mma_step<TH, OPS1>(a_ring + h * 8192, xbuf + h * (TM * 2048) + g * (TH * 2048),
-                                       &s_xs[h][g * (TH * 16) + n], s_ws[0][kb], s_ws[1][kb], acc, frag_lo, frag_hi,
+                    const float *row = xs_chunk ? &s_xc[(kb >> 2) & 1][g * (TH * 64) + n * 4 + (kb & 3)]
+                                                : &s_xs[h][g * (TH * 16) + n];
+                    mma_step<TH, OPS1>(a_ring + h * 8192, xbuf + h * (TM * 2048) + g * (TH * 2048), row,
+                                       xs_chunk ? 64 : 16, s_ws[0][kb], s_ws[1][kb], acc, frag_lo, frag_hi,
                                        [&](int i) { issue_op(kb + 2, (h + 2) % kStages, i); });
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -407,7 +424,7 @@ __global__ __launch_bounds__(512) void moe_tile_kernel(const TileParams s)
                     const int c0 = group_of(cg) << 6;
                     const float ws2 = s_w2s[(c0 >> 7) * n_ib + cib];
                     mma_step<THD, AOPS>(a_ring + h * 8192, aq + cib * (TMD * 2048) + g * (THD * 2048),
-                                        &s_sa[cib][g * (THD * 16) + n], ws2, ws2, accd, frag_lo, frag_hi,
+                                        &s_sa[cib][g * (THD * 16) + n], 16, ws2, ws2, accd, frag_lo, frag_hi,
                                         [&](int i) { issue2_op((h + 2) % kStages, i); });
                     advance2();
                     __builtin_amdgcn_sched_barrier(0);
@@ -682,6 +699,7 @@ hipError_t launch_tile(const MoeParams &p, int stages, void *workspace, hipStrea
     // on a queue, a down item's up/gate items were taken at least two rounds of the queue earlier
     s.lag = tunable(kTunTileLag, 64);
     s.w_nt = tunable(kTunTileNt, -1);
+    s.xs_chunk = (s.nkb % 4 == 0 && reinterpret_cast<uintptr_t>(p.x_scale) % 16 == 0) ? 1 : 0;
     if (s.lag < 1) s.lag = 1;
     const TileFn fn = pick(tm / 2);
     s.nh = token_parts(tm / 2, s.n_ib);

@@ -104,16 +104,16 @@ def test_nine_slices_row_blocks_above_32():
         assert_parity(run_op(P, *knobs, via="c_abi"), ref, f"nine slices {knobs}")
 
 
-def test_wide_kernel_fetches_activation_scales_both_ways():
-    """The wide kernel takes a token's activation scales four K blocks at a time where the row of scales allows 16-byte
-    loads (K / 128 a multiple of 4, x_scale 16-byte aligned) and one at a time otherwise: both ways against the oracle,
-    and bit for bit against each other on the same problem."""
+def test_prefill_kernels_fetch_activation_scales_both_ways():
+    """The tile and wide kernels take a token's activation scales four K blocks at a time where the row of scales allows
+    16-byte loads (K / 128 a multiple of 4, x_scale 16-byte aligned) and one at a time otherwise: both ways against the
+    oracle, and bit for bit against each other on the same problem."""
     for K in (384, 512, 640, 1024):
         shape = Shape("wx", E=6, top_k=4, K=K, I=256, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0)
         W = make_weights(shape, device=DEV, seed=K)
         P = make_problem(W, 300, seed=K)
         ref = oracle_out(P)
-        for knobs in ((128, 32, 8, 2), (48, 32, 8, 1)):
+        for knobs in ((128, 32, 8, 2), (48, 32, 8, 1), (128, 64, 4, 3), (64, 64, 4, 4)):
             print(f"case scale fetch K={K} knobs {knobs}", flush=True)
             a = run_op(P, *knobs, via="c_abi")
             m = assert_parity(a, ref, f"K={K} {knobs}")
