@@ -21,6 +21,7 @@ TunableSlot g_tunables[kTunCount] = {
     {"ALPHA_MOE_LAG", kTunableUnset},         {"ALPHA_MOE_GRID", kTunableUnset},
     {"ALPHA_MOE_TILE_GPS", kTunableUnset},    {"ALPHA_MOE_TILE_LAG", kTunableUnset},
     {"ALPHA_MOE_TILE_GRID", kTunableUnset},   {"ALPHA_MOE_TILE_NT", kTunableUnset},
+    {"ALPHA_MOE_WIDE_PP", kTunableUnset},
 };
 
 void load_tunables_once()

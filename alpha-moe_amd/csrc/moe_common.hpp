@@ -264,6 +264,7 @@ enum Tunable {
     kTunTileLag,       // ALPHA_MOE_TILE_LAG
     kTunTileGrid,      // ALPHA_MOE_TILE_GRID
     kTunTileNt,        // ALPHA_MOE_TILE_NT: non-temporal weight loads 1 always, 0 never
+    kTunWidePp,        // ALPHA_MOE_WIDE_PP: up/gate items of the wide kernel with the wavefronts of a SIMD half a step apart
     kTunCount
 };
 int tunable(Tunable which, int dflt);   // the override if one is set, else dflt

@@ -200,10 +200,10 @@ __device__ __forceinline__ void wide_step(const uint8_t *a_tiles, const uint8_t 
     }
 }
 
-// Half a step: token tiles T0 .. T0 + 3 of the wavefront against weight fragments already in registers.  Same
-// arithmetic and order as wide_step.
+// Half a step: token tiles T0 .. T0 + 3 of the wavefront (TS bytes apart in LDS) against weight fragments already in
+// registers.  Same arithmetic and order as wide_step.
 // The per-token factor of the wavefront's token tile t is row[t * row_a + (t >= 4 ? row_b : 0)].
-template <int T0, typename Issue>
+template <int T0, int TS, typename Issue>
 __device__ __forceinline__ void wide_half(const v8i (&a)[4], const uint8_t *b_tiles, const float *row, int row_a, int row_b,
                                           float sc0, float sc1, v4f (&acc)[4][8], int frag_lo, int frag_hi, int nt_w,
                                           Issue issue)
@@ -212,7 +212,7 @@ __device__ __forceinline__ void wide_half(const v8i (&a)[4], const uint8_t *b_ti
         return cat(*reinterpret_cast<const v4i *>(tile + frag_lo), *reinterpret_cast<const v4i *>(tile + frag_hi));
     };
     auto row_at = [&](int t) { return row[t * row_a + (t >= 4 ? row_b : 0)]; };
-    v8i b = read_tile(b_tiles + T0 * 4096);
+    v8i b = read_tile(b_tiles + T0 * TS);
     float f = row_at(T0);
 #pragma unroll
     for (int t = T0; t < T0 + 4; t++) {
@@ -220,7 +220,7 @@ __device__ __forceinline__ void wide_half(const v8i (&a)[4], const uint8_t *b_ti
         v8i b_next = b;
         float f_next = f;
         if (t + 1 < T0 + 4) {
-            b_next = read_tile(b_tiles + (t + 1) * 4096);
+            b_next = read_tile(b_tiles + (t + 1) * TS);
             f_next = row_at(t + 1);
         }
         if (t < nt_w) {
@@ -243,6 +243,141 @@ __device__ __forceinline__ void wide_half(const v8i (&a)[4], const uint8_t *b_ti
         b = b_next;
         f = f_next;
     }
+}
+
+// A whole step of a wavefront that has the matrix pipe to itself: its token tiles (TS bytes apart in LDS) against weight
+// fragments in registers, same arithmetic and order per accumulator as wide_step.  A lone wavefront issues one
+// instruction every four cycles and a matrix instruction occupies the pipe for 32, so a token tile (four matrix
+// instructions) has 32 issue slots and the stream must be straight-line and free of wait states to keep the pipe fed:
+//  - a product is scaled into its accumulator D matrix instructions after its own (a vector instruction may read a
+//    product 11 slots after the matrix instruction was issued; a group of one matrix instruction and four
+//    multiply-adds is 5), and the queue of D products lives on from one step to the next: it is cleared before an
+//    item's first step and drained after its last (wide_queue_drain);
+//  - the tiles run from the top down and only in blocks of four: tiles 7 .. 4 when the wavefront has more than four
+//    live tiles, then tiles 3 .. 0, so a step always ends with tile 0 and the products a step finds in the queue are
+//    those of tile 0.  A dead tile of a block is multiplied like a live one (whatever its LDS holds; nobody reads a dead
+//    tile's accumulators);
+//  - the first tile's operands are read at the start of the step (wide_top_read), every other tile's while the tile
+//    before it is multiplied; the weight-block factors and the weight fragments are in registers before the barrier
+//    that starts the step.
+// The operand reads are written as instructions the compiler knows nothing about, and waited for by hand: it would
+// wait for ALL outstanding LDS reads before a tile's first matrix instruction, the next tile's (just issued) included,
+// which puts an LDS round trip into every other tile.  LDS reads complete in order, so "at most the three reads just
+// issued are outstanding" is what a tile needs.
+template <int OFF>
+__device__ __forceinline__ v4i lds_read16_raw(unsigned addr)
+{
+    v4i v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    return v;
+}
+__device__ __forceinline__ float lds_read4_raw(unsigned addr)
+{
+    float v;
+    asm volatile("ds_read_b32 %0, %1" : "=v"(v) : "v"(addr));
+    return v;
+}
+template <int N>
+__device__ __forceinline__ void lds_landed_but(v4i &lo, v4i &hi, float &f)
+{
+    asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(lo), "+v"(hi), "+v"(f) : "n"(N));
+}
+
+// operands of the first tile of a step: tile 7 (upper) or 3
+template <int TS>
+__device__ __forceinline__ void wide_top_read(const uint8_t *b_tiles, const float *row, int row_a, int frag_lo, int frag_hi,
+                                              bool upper, v4i &b_lo, v4i &b_hi, float &f)
+{
+    const unsigned a_lo = (uint32_t)(uintptr_t)b_tiles + (unsigned)frag_lo, a_hi = (uint32_t)(uintptr_t)b_tiles + (unsigned)frag_hi;
+    const unsigned a_f = (uint32_t)(uintptr_t)row, f_stride = 4u * (unsigned)row_a;
+    if (upper) {
+        b_lo = lds_read16_raw<7 * TS>(a_lo);
+        b_hi = lds_read16_raw<7 * TS>(a_hi);
+        f = lds_read4_raw(a_f + 7u * f_stride);
+    } else {
+        b_lo = lds_read16_raw<3 * TS>(a_lo);
+        b_hi = lds_read16_raw<3 * TS>(a_hi);
+        f = lds_read4_raw(a_f + 3u * f_stride);
+    }
+}
+
+template <int TS, int D>
+__device__ __forceinline__ void wide_tiles8(const v8i (&a)[4], const uint8_t *b_tiles, const float *row, int row_a, float sc0,
+                                            float sc1, v4f (&acc)[4][8], int frag_lo, int frag_hi, bool upper, v4i &b_lo,
+                                            v4i &b_hi, float &f, v4f (&prod)[D], float (&fac)[D])
+{
+    static_assert(D >= 1 && D <= 3, "queue depth");
+    static_assert(7 * TS < 65536, "tile offsets are instruction immediates");
+    const unsigned a_lo = (uint32_t)(uintptr_t)b_tiles + (unsigned)frag_lo, a_hi = (uint32_t)(uintptr_t)b_tiles + (unsigned)frag_hi;
+    const unsigned a_f = (uint32_t)(uintptr_t)row, f_stride = 4u * (unsigned)row_a;
+    // tile t; the tile multiplied before it was tile `before` (of this step, or tile 0 of the step before)
+    auto tile = [&](auto tc, auto bc) {
+        constexpr int t = decltype(tc)::value, before = decltype(bc)::value;
+        v4i n_lo = b_lo, n_hi = b_hi;
+        float n_f = f;
+        if constexpr (t > 0) {
+            n_lo = lds_read16_raw<(t > 0 ? t - 1 : 0) * TS>(a_lo);
+            n_hi = lds_read16_raw<(t > 0 ? t - 1 : 0) * TS>(a_hi);
+            n_f = lds_read4_raw(a_f + (unsigned)(t - 1) * f_stride);
+            lds_landed_but<3>(b_lo, b_hi, f);
+        } else {
+            lds_landed_but<0>(b_lo, b_hi, f);
+        }
+        const v8i b = cat(b_lo, b_hi);
+        const float p0 = f * sc0, p1 = f * sc1;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const v4f cur = mfma_fp8(a[k], b);
+            __builtin_amdgcn_sched_barrier(0);
+            // the oldest product of the queue: D matrix instructions back
+            v4f &dst = k >= D ? acc[k - D][t] : acc[4 - D + k][before];
+            dst += prod[0] * fac[0];
+            asm volatile("" : "+v"(dst));
+#pragma unroll
+            for (int i = 0; i + 1 < D; i++) {
+                prod[i] = prod[i + 1];
+                fac[i] = fac[i + 1];
+            }
+            prod[D - 1] = cur;
+            fac[D - 1] = (k & 1) ? p1 : p0;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        b_lo = n_lo;
+        b_hi = n_hi;
+        f = n_f;
+    };
+    using std::integral_constant;
+    if (upper) {
+        tile(integral_constant<int, 7>{}, integral_constant<int, 0>{});
+        tile(integral_constant<int, 6>{}, integral_constant<int, 7>{});
+        tile(integral_constant<int, 5>{}, integral_constant<int, 6>{});
+        tile(integral_constant<int, 4>{}, integral_constant<int, 5>{});
+        tile(integral_constant<int, 3>{}, integral_constant<int, 4>{});
+    } else {
+        tile(integral_constant<int, 3>{}, integral_constant<int, 0>{});
+    }
+    tile(integral_constant<int, 2>{}, integral_constant<int, 3>{});
+    tile(integral_constant<int, 1>{}, integral_constant<int, 2>{});
+    tile(integral_constant<int, 0>{}, integral_constant<int, 1>{});
+}
+
+template <int D>
+__device__ __forceinline__ void wide_queue_clear(v4f (&prod)[D], float (&fac)[D])
+{
+#pragma unroll
+    for (int i = 0; i < D; i++) {
+        prod[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+        fac[i] = 0.f;
+    }
+}
+
+// after an item's last step: the queue holds the last D products of tile 0
+template <int D>
+__device__ __forceinline__ void wide_queue_drain(v4f (&acc)[4][8], v4f (&prod)[D], float (&fac)[D])
+{
+#pragma unroll
+    for (int i = 0; i < D; i++) acc[4 - D + i][0] += prod[i] * fac[i];
 }
 
 // "At most n of this wavefront's loads are still outstanding", n known only at run time (the same for all lanes).
@@ -270,6 +405,12 @@ __device__ __forceinline__ void wait_pending(int n)
     }
 }
 
+// Products in flight between a matrix instruction and its scaled accumulate in the ping-pong loop: two leave one wait
+// state per matrix instruction and keep the loops free of register spills (three would leave none, and spill).
+constexpr int kPpDepth = 2;
+
+// PP: the up/gate items run the two wavefronts of a SIMD half a step apart (see up_item).
+template <bool PP>
 __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
 {
     constexpr int THREADS = 512;
@@ -380,6 +521,151 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
         const int nt_w = n_tiles > g ? (n_tiles - g + 1) >> 1 : 0;
         const int unit = mc.mb0 * n_ib + ib;
         if (n_tiles > 0) {
+            if constexpr (PP) {
+                // Ping-pong: the wavefronts with g = 0 and those with g = 1 - the two wavefronts of every SIMD - run half a
+                // step apart.  In one half step a wavefront multiplies (the matrix instructions of a K step with their
+                // scaled accumulates and operand reads, nothing else: wide_tiles8), in the other it issues its loads,
+                // waits for the batch before, and reads the weight fragments and factors of its next step; a barrier ends
+                // each half step.  So on every SIMD one wavefront is at its memory instructions while the other has the
+                // matrix pipe to itself (matrix and memory instructions of different wavefronts overlap completely; those
+                // of one wavefront, or of two in the same phase, add up).
+                //   half step 2 kb:     g = 0 multiplies step kb          g = 1 loads odd token tiles of step kb + 1
+                //   half step 2 kb + 1: g = 0 loads weights and even      g = 1 multiplies step kb
+                //                       token tiles of step kb + 2
+                // Weights of step kb: ring slot kb & 1 (its fragments are in everybody's registers one half step before
+                // it is refilled).  Token tiles: the even tiles of step kb are half 2 kb of a stream, the odd ones half
+                // 2 kb + 1; half hh sits in quarter hh & 3 of the token region and is refilled with half hh + 4 one half
+                // step after its use.  Every load is issued three half steps before its first use.
+                const bool xs_chunk = s.xs_chunk != 0;
+                const int row_a = xs_chunk ? 128 : 16;
+                float *s_xs4 = &s_xs[0][0];   // per-step scales (not chunked): [half & 3][tile of the half][token]
+                // this wavefront's two token tiles of its half: e = 2 w, 2 w + 1 (token tile 2 e + g)
+                unsigned x_off[2][2], xs_off[2];
+                bool x_live[2];
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const int tt = 2 * (2 * w + j) + g;
+                    x_live[j] = tt < n_tiles;
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const int tk = s_tok[tt * 16 + 8 * h + ld_row];
+                        x_off[j][h] = (unsigned)(tk < 0 ? 0 : tk) * (unsigned)K + ld_chunk[h];
+                    }
+                    const int tk = s_tok[tt * 16 + n];
+                    xs_off[j] = (unsigned)(tk < 0 ? 0 : tk) * (unsigned)nkb;
+                }
+                // weights (g = 0 only): all four tiles of pair w; tile a = (32-row group a / 2, gate | up a % 2)
+                unsigned w_voff[2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) w_voff[h] = (unsigned)((ib * 256 + w * 64 + ld_row) * p.w_rs) + ld_chunk[h];
+                const uint8_t *wexp = p.w + (size_t)mc.e * p.N * K;
+                const bool nt = mc.lone;
+                // the wavefront's loads of step kn; returns how many instructions went out
+                auto issue_batch = [&](int kn) {
+                    int cnt = 0;
+                    if (kn >= nkb) return cnt;
+                    if (g == 0) {
+#pragma unroll
+                        for (int a = 0; a < 4; a++)
+#pragma unroll
+                            for (int h = 0; h < 2; h++) {
+                                const uint8_t *src = wexp + (size_t)kn * p.w_ks + (size_t)((a >> 1) * 32 + h * 16 + 8 * (a & 1)) * p.w_rs;
+                                uint8_t *dst = a_ring + (kn & 1) * kWStageA + w * 8192 + a * 2048 + h * 1024;
+                                if (nt) dma16_sv<2>(src, w_voff[h], dst);
+                                else dma16_sv<0>(src, w_voff[h], dst);
+                                cnt++;
+                            }
+                    }
+                    const int hh = 2 * kn + g;
+                    uint8_t *xq = xbuf + (hh & 3) * 16384;
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        if (!x_live[j]) continue;
+                        const int e = 2 * w + j;
+#pragma unroll
+                        for (int h = 0; h < 2; h++)
+                            dma16_sv<0>(p.x + (size_t)kn * 128, x_off[j][h], xq + e * 2048 + h * 1024);
+                        cnt += 2;
+                        if (xs_chunk) {
+                            if ((kn & 3) == 0) {
+                                if (lane < 16) dma16_sv<0>(p.x_scale + kn, xs_off[j] * 4u, &s_xc[(kn >> 2) & 1][(2 * e + g) * 64]);
+                                cnt++;
+                            }
+                        } else {
+                            if (lane < 16) dma4_sv<0>(p.x_scale + kn, xs_off[j] * 4u, s_xs4 + (hh & 3) * 128 + e * 16);
+                            cnt++;
+                        }
+                    }
+                    return cnt;
+                };
+                v8i a[4];
+                auto read_a = [&](int kb) {
+                    const uint8_t *a_tiles = a_ring + (kb & 1) * kWStageA + w * 8192;
+#pragma unroll
+                    for (int k = 0; k < 4; k++)
+                        a[k] = cat(*reinterpret_cast<const v4i *>(a_tiles + k * 2048 + frag_lo),
+                                   *reinterpret_cast<const v4i *>(a_tiles + k * 2048 + frag_hi));
+                    // waited for here: a wait of the compiler's in the multiply phase would also cover the operand reads
+                    // in flight there, which it does not know of
+                    asm volatile("" ::"v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]));
+                };
+                const bool upper = nt_w > 4;
+                v4i top_lo, top_hi;   // operands of the first tile of the next step, and its weight-block factors
+                float top_f, top_sc0, top_sc1;
+                v4f q_prod[kPpDepth];
+                float q_fac[kPpDepth];
+                wide_queue_clear(q_prod, q_fac);
+                auto row_of = [&](int kb) {
+                    return xs_chunk ? &s_xc[(kb >> 2) & 1][g * 64 + n * 4 + (kb & 3)] : s_xs4 + ((2 * kb + g) & 3) * 128 + n;
+                };
+                // before the barrier that starts a multiply phase: the step's weight-block factors
+                auto read_sc = [&](int kb) {
+                    top_sc0 = s_ws[0][kb];
+                    top_sc1 = s_ws[1][kb];
+                    asm volatile("" ::"v"(top_sc0), "v"(top_sc1));   // (as in read_a)
+                };
+                auto multiply = [&](int kb) {
+                    if (nt_w > 0) {
+                        wide_top_read<2048>(xbuf + ((2 * kb + g) & 3) * 16384, row_of(kb), row_a, frag_lo, frag_hi, upper, top_lo,
+                                            top_hi, top_f);
+                        wide_tiles8<2048, kPpDepth>(a, xbuf + ((2 * kb + g) & 3) * 16384, row_of(kb), row_a, top_sc0, top_sc1, acc,
+                                                    frag_lo, frag_hi, upper, top_lo, top_hi, top_f, q_prod, q_fac);
+                    }
+                };
+                clear_acc();
+                if (g == 0) {
+                    issue_batch(0);
+                    const int c1 = issue_batch(1);
+                    wait_pending(c1);
+                    read_a(0);
+                    read_sc(0);
+                    lds_barrier();
+                    for (int kb = 0; kb < nkb; kb++) {
+                        multiply(kb);
+                        lds_barrier();
+                        const int cnt = issue_batch(kb + 2);
+                        wait_pending(cnt);   // the loads of step kb + 1 have landed
+                        if (kb + 1 < nkb) {
+                            read_a(kb + 1);
+                            read_sc(kb + 1);
+                        }
+                        lds_barrier();
+                    }
+                } else {
+                    issue_batch(0);
+                    lds_barrier();
+                    for (int kb = 0; kb < nkb; kb++) {
+                        const int cnt = issue_batch(kb + 1);
+                        wait_pending(cnt);   // the odd token tiles of step kb have landed
+                        read_a(kb);          // (its weights: g = 0 waited for them before the barrier)
+                        read_sc(kb);
+                        lds_barrier();
+                        multiply(kb);
+                        lds_barrier();
+                    }
+                }
+                wide_queue_drain(acc, q_prod, q_fac);
+            } else {
             // token-tile gather: wavefront v loads tiles v and v + 8
             const bool xs_chunk = s.xs_chunk != 0;
             const int row_a = xs_chunk ? 128 : 64, row_b = xs_chunk ? 0 : -240;
@@ -476,7 +762,7 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
                         const float *row = xs_chunk ? &s_xc[(kb >> 2) & 1][g * 64 + n * 4 + (kb & 3)] : &s_xs[h][row_off];
                         // loads of the step, five or so per half: weights of step kb + 2 (halves 0, 1 | 2, 3), the
                         // second token half of step kb + 1 | the first token half of step kb + 2
-                        wide_half<0>(a, xbuf + h * kWStageX + g * 2048, row, row_a, row_b, sc0, sc1, acc, frag_lo,
+                        wide_half<0, 4096>(a, xbuf + h * kWStageX + g * 2048, row, row_a, row_b, sc0, sc1, acc, frag_lo,
                                      frag_hi, nt_w, [&](int t) {
                                          if (kb + 2 < nkb && (t & 1) == 0) issue_a_op(kb + 2, h, t >> 1);
                                          if (kb + 1 < nkb) {
@@ -487,7 +773,7 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
                         mark_hi[h ^ 1] = issued;
                         wait_pending(issued - mark_hi[h]);
                         lds_barrier();   // everybody is done with token tiles 0..7; tiles 8..15 have landed
-                        wide_half<4>(a, xbuf + h * kWStageX + g * 2048, row, row_a, row_b, sc0, sc1, acc, frag_lo,
+                        wide_half<4, 4096>(a, xbuf + h * kWStageX + g * 2048, row, row_a, row_b, sc0, sc1, acc, frag_lo,
                                      frag_hi, nt_w, [&](int t) {
                                          if (kb + 2 < nkb) {
                                              if ((t & 1) == 0) issue_a_op(kb + 2, h, 2 + ((t - 4) >> 1));
@@ -499,6 +785,7 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
                         mark_lo[h] = issued;
                     }
                 }
+            }
             }
             wait_vmcnt<0>();
 
@@ -789,8 +1076,11 @@ hipError_t allow_dynamic_lds()
     if (err != hipSuccess) return err;
     std::lock_guard<std::mutex> lock(mu);
     if (dev >= 0 && dev < 64 && done[dev]) return hipSuccess;
-    err = hipFuncSetAttribute(reinterpret_cast<const void *>(moe_wide_kernel),
+    err = hipFuncSetAttribute(reinterpret_cast<const void *>(moe_wide_kernel<false>),
                               hipFuncAttributeMaxDynamicSharedMemorySize, kWDynLds);
+    if (err == hipSuccess)
+        err = hipFuncSetAttribute(reinterpret_cast<const void *>(moe_wide_kernel<true>),
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kWDynLds);
     if (err == hipSuccess && dev >= 0 && dev < 64) done[dev] = true;
     return err;
 }
@@ -869,7 +1159,14 @@ hipError_t launch_wide(const MoeParams &p, int stages, void *workspace, hipStrea
     int grid = tunable(kTunTileGrid, cus);
     if (grid > items) grid = (int)((items + 7) / 8 * 8);
     if (grid < 8) grid = 8;
-    hipLaunchKernelGGL(moe_wide_kernel, dim3((unsigned)grid), dim3(512), kWDynLds, stream, s);
+    // The ping-pong up/gate loop multiplies a wavefront's token tiles in blocks of four, dead ones included, and so pays
+    // off when an expert's rows fill its 256-row blocks: by default it is used from 192 routed rows per expert on
+    // average (measured: 2 - 3 % on whole calls there; slower below).  The result does not depend on the choice.
+    const int pp_default = (int64_t)p.M * p.top_k >= (int64_t)192 * p.E ? 1 : 0;
+    if (tunable(kTunWidePp, pp_default) != 0)
+        hipLaunchKernelGGL(moe_wide_kernel<true>, dim3((unsigned)grid), dim3(512), kWDynLds, stream, s);
+    else
+        hipLaunchKernelGGL(moe_wide_kernel<false>, dim3((unsigned)grid), dim3(512), kWDynLds, stream, s);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
     RowsReduce r;

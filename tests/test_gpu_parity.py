@@ -129,6 +129,38 @@ def test_prefill_kernels_fetch_activation_scales_both_ways():
             assert torch.equal(a, b), (K, knobs)
 
 
+def test_wide_kernel_up_loop_variants_give_the_same_bits():
+    """The wide kernel has two forms of its up/gate loop: both wavefronts of a SIMD in step, or half a step apart (one
+    multiplies a whole step alone, token tiles in blocks of four from the top down with a queue of pending products
+    that lives across steps, while the other loads).  ALPHA_MOE_WIDE_PP picks one (unset: by rows per expert).  Both
+    against the oracle and bit for bit against each other, over: one to sixteen live token tiles in a block and blocks
+    whose second wavefront of a pair has none; one, two, three, four and eight K steps (the loop's prologue issues
+    two steps of loads; activation scales are fetched four steps at a time from K = 512 on and singly otherwise, also
+    from a row of scales that is not 16-byte aligned); experts with one block of rows and with several."""
+    for K, M in ((128, 150), (256, 300), (384, 40), (512, 700), (1024, 300), (512, 9), (640, 150)):
+        shape = Shape("pp", E=6, top_k=4, K=K, I=256, shared_expert=False, routing="softmax_renorm", scaling_factor=1.0)
+        W = make_weights(shape, device=DEV, seed=K + M)
+        P = make_problem(W, M, seed=K + M)
+        ref = oracle_out(P)
+        for knobs in ((128, 32, 8, 2), (48, 32, 8, 1)):
+            outs = []
+            for pp in (0, 1):
+                print(f"case up loop K={K} M={M} knobs {knobs} ALPHA_MOE_WIDE_PP={pp}", flush=True)
+                with tunables(ALPHA_MOE_WIDE_PP=pp):
+                    outs.append(run_op(P, *knobs, via="c_abi"))
+                assert_parity(outs[-1], ref, f"K={K} M={M} {knobs} pp={pp}")
+            assert torch.equal(outs[0], outs[1]), (K, M, knobs)
+            if K == 512 and M == 700:
+                aligned = P.x_scale
+                raw = torch.empty(aligned.numel() + 1, dtype=torch.float32, device=DEV)
+                raw[1:].copy_(aligned.flatten())
+                P.x_scale = raw[1:].view_as(aligned)
+                with tunables(ALPHA_MOE_WIDE_PP=1):
+                    b = run_op(P, *knobs, via="c_abi")
+                P.x_scale = aligned
+                assert torch.equal(outs[0], b), (K, M, knobs, "unaligned scales")
+
+
 def test_store_variant_fallback_kernel():
     """129 K blocks are more than the tile and wide kernels take: the fallback kernel serves the call, and its store
     variant overwrites too."""
