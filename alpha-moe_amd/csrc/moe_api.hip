@@ -326,4 +326,4 @@ extern "C" const char *alpha_moe_status_string(int status)
     }
 }
 
-extern "C" const char *alpha_moe_version(void) { return "0.5"; }
+extern "C" const char *alpha_moe_version(void) { return "0.6"; }

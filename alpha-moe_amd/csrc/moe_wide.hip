@@ -545,7 +545,7 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
 #pragma unroll
                 for (int j = 0; j < 2; j++) {
                     const int tt = 2 * (2 * w + j) + g;
-                    x_live[j] = tt < n_tiles;
+                    x_live[j] = rfl(tt < n_tiles ? 1 : 0) != 0;   // (the same in all lanes; a scalar for the compiler too)
 #pragma unroll
                     for (int h = 0; h < 2; h++) {
                         const int tk = s_tok[tt * 16 + 8 * h + ld_row];
@@ -596,7 +596,7 @@ __global__ __launch_bounds__(512) void moe_wide_kernel(const WideParams s)
                             cnt++;
                         }
                     }
-                    return cnt;
+                    return rfl(cnt);
                 };
                 v8i a[4];
                 auto read_a = [&](int kb) {
